@@ -230,6 +230,101 @@ class StreamScaleSpec:
 
 
 @dataclass(frozen=True)
+class ChunkAttentionSpec:
+    """Grouped-query attention inside chunks of positions: with ``chunk`` = c, a query at position i sees the keys
+    j <= i with i // c == j // c, chunks counted from the request's start (None: all earlier keys).  Keys have
+    ``head_dim`` numbers, values ``v_head_dim``; all four projections have biases if ``bias``.
+    ``qk_norm``: None, "head" (RMS norm of every q and k head with one weight of the head's size for all heads) or
+    "whole" (RMS norm over all heads of q, and of k, at once, a weight per coordinate), before the rotation.
+    ``values_from_keys``: there is no value projection; the values are the keys as projected, before their norm.
+    ``value_norm_eps``: every value head is divided by its root mean square (no weight).
+    ``value_blend``: None; "source": the values (after their norm) are also left for later layers of the step;
+    "blend": v <- (1 - l) v + l v_source with l a tensor of the layer; what is blended is what is cached.
+    ``distance_bias_rows`` = B > 0: a table [B, heads] is added to the scaled scores by distance n = i - j: row n
+    for n < B // 2, else min(B - 1, B // 2 + floor(log(n / (B // 2)) / log(far / (B // 2)) * (B - B // 2))) with
+    far = ``distance_bias_far``.  ``talking_heads``: the heads' scores are then mixed by a matrix [heads, heads]
+    before the softmax.  ``names``: tensors of q, k, v, output projection; the others by the suffixes below."""
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    scale: float
+    chunk: Optional[int] = None
+    bias: bool = False
+    qk_norm: Optional[str] = None
+    qk_norm_eps: float = 0.0
+    values_from_keys: bool = False
+    value_norm_eps: Optional[float] = None
+    value_blend: Optional[str] = None
+    distance_bias_rows: int = 0
+    distance_bias_far: float = 0.0
+    talking_heads: bool = False
+    position: Optional[object] = None
+    names: Tuple[str, str, str, str] = ("q", "k", "v", "o")
+    bias_suffix: str = ".b"
+    norm_suffix: str = ".norm"
+    blend_name: str = "vmix"
+    distance_bias_name: str = "rel"
+    talk_name: str = "talk"
+    kind: str = "chunk_attention"
+
+
+@dataclass(frozen=True)
+class ShiftedDecaySpec:
+    """A recurrence per head over a state S [head_dim][head_dim] whose inputs are blends of a token x and the token
+    before it x' (zeros before the first): m_s = x + (x' - x) mu_s for s in r, k, v, g, w.  r, k, v = W m; gate =
+    silu(W_g m_g); decay w = exp(-exp(W_2 tanh(W_1 m_w) + w0)) per key channel (W_1 has ``decay_rank`` rows);
+    o_t = (S + diag(u) k_t v_t^T)^T r_t, then S <- diag(w_t) S + k_t v_t^T; each head's o divided by its root mean
+    square, times a weight, times the gate, then the output projection."""
+    num_heads: int
+    head_dim: int
+    decay_rank: int
+    norm_eps: float
+    kind: str = "shifted_decay"
+
+
+@dataclass(frozen=True)
+class DecayedLinearSpec:
+    """Linear attention with one decay per head: q, k = silu(W x) with ``head_dim`` numbers a head, v = silu(W x)
+    with ``v_head_dim``; S <- decay_h S + k_t v_t^T, o_t = S^T q_t; all heads' o normed together (RMS norm with a
+    weight), times sigmoid(W_g x), then the output projection."""
+    num_heads: int
+    head_dim: int
+    v_head_dim: int
+    decay: Tuple[float, ...]
+    norm_eps: float
+    kind: str = "decayed_linear"
+
+
+@dataclass(frozen=True)
+class SideBySideMixerSpec:
+    """Two mixers that read the same input; the result is left_scale * left + right_scale * right.  Their tensors
+    lie under ``names`` inside the mixer.  At most one of them keeps keys and values and at most one a state."""
+    left: object
+    right: object
+    left_scale: float
+    right_scale: float
+    names: Tuple[str, str] = ("left", "right")
+    kind: str = "side_by_side"
+
+
+@dataclass(frozen=True)
+class GeluMLPSpec:
+    """down(gelu(up x)) with the exact gelu 0.5 z (1 + erf(z / sqrt 2)), no biases."""
+    intermediate_size: int
+    names: Tuple[str, str] = ("up", "down")
+    kind: str = "gelu_mlp"
+
+
+@dataclass(frozen=True)
+class LogitSoftcapSpec:
+    """logits <- cap * tanh(logits / cap); no tensors."""
+    cap: float
+    prefix: str = ""
+    kind: str = "logit_softcap"
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One pre-norm residual block: x += mixer(norm(x)); x += ffn(norm(x)).
 

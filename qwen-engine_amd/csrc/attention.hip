@@ -91,7 +91,7 @@ extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* ca
                                         float scale, int window, int keep_first, int sink, int groups, int seg_keys,
                                         int max_keys, int keys_row, void* workspace, long workspace_bytes,
                                         hipStream_t stream) {
-    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && keep_first >= 0 &&
+    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && keep_first >= 0 &&
                workspace_bytes >= 0, "prefill attention: bad sizes");
     return qe_attention_prefill(q, out, cache, tiles, num_tiles, positions, tok_seq, block_table, max_blocks,
                                 Hq, Hkv, D, P, scale, window, groups, seg_keys, max_keys, keys_row, workspace,
@@ -106,7 +106,7 @@ extern "C" int qe_attention(const void* q, void* out, const void* cache, const i
                             int sink, int dt_a, hipStream_t stream) {
     QE_REQUIRE(n_tokens >= 0 && Hq > 0 && Hkv > 0 && D > 0 && P > 0 && max_blocks > 0, "attention: bad sizes");
     QE_REQUIRE(Hq % Hkv == 0, "attention: %d query heads are no multiple of %d key/value heads", Hq, Hkv);
-    QE_REQUIRE(window >= 0 && keep_first >= 0, "attention: negative window or kept keys");
+    QE_REQUIRE(keep_first >= 0 && (window >= 0 || keep_first == 0), "attention: kept first keys go with a window of the last keys");
     if (n_tokens == 0) return 0;
     return qe_attention_generic(q, out, cache, positions, tok_seq, block_table, max_blocks, tokens, n_tokens,
                                 Hq, Hkv, D, P, scale, window, keep_first, sink, dt_a, stream);
@@ -144,7 +144,7 @@ extern "C" int qe_attention_decode_fused_run(const void* qkv, void* out, void* c
                                              int Hq, int Hkv, int D, int P, float scale, int window,
                                              int max_position, int split_keys, void* workspace,
                                              long workspace_bytes, hipStream_t stream) {
-    QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && max_position >= 0, "decode attention: bad sizes");
+    QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && max_position >= 0, "decode attention: bad sizes");
     return qe_attention_decode_fused(qkv, out, cache, dec_tokens, n_dec, positions, tok_seq, block_table,
                                      max_blocks, shared_keys, slots, q_w, k_w, eps, table, Hq, Hkv, D, P, scale, window,
                                      max_position, split_keys, workspace, (size_t)workspace_bytes, stream);
@@ -156,7 +156,7 @@ extern "C" int qe_attention_decode_run(const void* q, void* out, const void* cac
                                        int Hq, int Hkv, int D, int P, float scale, int window, int keep_first, int sink,
                                        int max_position, int split_keys, void* workspace, long workspace_bytes,
                                        hipStream_t stream) {
-    QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && keep_first >= 0 && max_position >= 0,
+    QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && keep_first >= 0 && max_position >= 0,
                "decode attention: bad sizes");
     return qe_attention_decode(q, out, cache, dec_tokens, n_dec, positions, tok_seq, block_table, max_blocks,
                                shared_keys, Hq, Hkv, D, P, scale, window, keep_first, sink, max_position, split_keys,

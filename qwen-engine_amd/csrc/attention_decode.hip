@@ -25,7 +25,7 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const int G = Hq / Hkv;
     const int t = dec_tokens ? dec_tokens[di] : di;       // (no list: every row, in order)
     const int p = positions[t];
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int lo = first_seen_key(p, window);
     const int k_begin = max(split * SPLIT, lo);
     const int k_end = min((split + 1) * SPLIT, p + 1);
     // the request's kept first keys that lie behind the window, as far as they are this split's: [split * SPLIT, kf)
@@ -202,7 +202,7 @@ __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
     const int G = Hq / Hkv;
     const int t = dec_tokens ? dec_tokens[di] : di;       // (no list: every row, in order)
     const int p = positions[t];
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int lo = first_seen_key(p, window);
     const bool own = split == p / SPLIT;                   // this wave takes the token's own key and value
     const int k_begin = max(split * SPLIT, lo);
     const int k_end = min((split + 1) * SPLIT, p);         // cached keys: the token's own is not among them

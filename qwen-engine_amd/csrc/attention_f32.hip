@@ -49,7 +49,7 @@ __global__ __launch_bounds__(64 * F32_WAVES) void attention_f32_kernel(
     const int head = kvh * G + hg * 16 + n;
     const bool head_ok = hg * 16 + n < G;
     const int p = positions[t];
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int lo = first_seen_key(p, window);
     const int* bt = block_table + (long)tok_seq[t] * max_blocks;
     const long page_stride = 2L * Hkv * P * D;
     const bool vec_v = (P & 3) == 0;                      // four consecutive keys of a value row lie in one page, aligned

@@ -35,7 +35,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const int kvh = h / (Hq / Hkv);
     const int p_own = positions[t];
     const int* bt = block_table + (long)tok_seq[t] * max_blocks;
-    const int lo = (window > 0 && p_own - window + 1 > 0) ? p_own - window + 1 : 0;
+    const int lo = first_seen_key(p_own, window);
     const long page_stride = 2L * Hkv * P * D;
 
     const TA* qrow = q + (t * Hq + h) * D;

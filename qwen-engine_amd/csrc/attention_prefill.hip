@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
 #pragma unroll
     for (int j = 1; j < 4; ++j) if (bt4[2 * j + 1] > 0) last = j;
     const int p_block = positions[row_first];
-    int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
+    int kmin = first_seen_key(p_block, window);
     int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
     // the request's kept first keys that lie behind the block's window: [0, kfb) (never together with segments)
     const int kfb = keep_first < kmin ? keep_first : kmin;
@@ -171,14 +171,14 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     const int row = wave_on ? row0 + (rr < cnt ? rr : cnt - 1) : row_first;   // columns beyond the tile repeat its last row
     const int p = positions[row];
     const int hi = p + 1;
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int lo = first_seen_key(p, window);
     const int p_first = positions[wave_on ? row0 : row_first];
-    const int k_start = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    const int k_start = first_seen_key(p_first, window);
     const int k_stop = wave_on ? p_first + cnt : 0;       // positions of a tile's rows are consecutive
     // keys every column of the wave sees without a limit: [all_lo, all_hi)
     const int p_last = p_first + cnt - 1;
     const int all_hi = p_first + 1;
-    const int all_lo = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+    const int all_lo = first_seen_key(p_last, window);
 
     bf16x8 qreg[D / 16];
 #pragma unroll
@@ -447,7 +447,7 @@ __global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
 #pragma unroll
     for (int j = 1; j < 4; ++j) if (bt4[2 * j + 1] > 0) last = j;
     const int p_block = positions[row_first];
-    const int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
+    const int kmin = first_seen_key(p_block, window);
     const int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
     const int seg_keys = segment_keys(seg_param, positions, keys_row);
     if (seg_keys <= 0) return;                             // nothing was cut

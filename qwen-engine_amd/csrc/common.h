@@ -36,6 +36,15 @@ __device__ __forceinline__ bf16_t float_to_bf16(float f) {
     return r;
 }
 
+// The first key a query at position p sees: window > 0, the last `window` keys (its own included);
+// window < 0, chunks of -window positions counted from the sequence's start: the first position of its
+// own chunk; 0: every key.  Both limits never move back as p grows.
+__device__ __forceinline__ int first_seen_key(int p, int window) {
+    if (window > 0) return p - window + 1 > 0 ? p - window + 1 : 0;
+    if (window < 0) return p / (-window) * (-window);
+    return 0;
+}
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static __device__ __forceinline__ float load(const float* p) { return *p; }

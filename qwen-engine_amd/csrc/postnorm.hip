@@ -1,4 +1,5 @@
-// Norm after the residual sum, with one gain for all coordinates, on the 32-bit stream:
+// Norm after the residual sum on the 32-bit stream, with one gain for all coordinates (gain_n = 1) or one
+// per coordinate (gain_n = H):
 //   z = alpha * x + (delta_0 + delta_1 + ...);   x <- g * z * rsqrt(mean(z^2) + eps)
 // and, if asked for, a copy of the new x in the activation type (what the next products read).
 // delta holds n_delta tensors [T, H] one after the other (one branch output, or partial products
@@ -13,7 +14,7 @@
 // reads it back.
 template <typename TA, typename TD>
 __global__ void postnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_delta, long delta_stride,
-                                float alpha, const float* __restrict__ gain, float eps, TA* __restrict__ act,
+                                float alpha, const float* __restrict__ gain, int gain_n, float eps, TA* __restrict__ act,
                                 int H) {
     __shared__ float red[16];
     const long r = blockIdx.x;
@@ -31,9 +32,9 @@ __global__ void postnorm_kernel(float* __restrict__ x, const TD* __restrict__ de
         ss += z * z;
     }
     ss = block_sum(ss, red);
-    const float f = rsqrtf(ss / (float)H + eps) * gain[0];
+    const float f = rsqrtf(ss / (float)H + eps) * (gain_n == 1 ? gain[0] : 1.f);
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
-        const float v = xr[c] * f;
+        const float v = gain_n == 1 ? xr[c] * f : xr[c] * f * gain[c];
         xr[c] = v;
         if (act) Elem<TA>::store(act + r * H + c, v);
     }
@@ -44,7 +45,7 @@ __global__ void postnorm_kernel(float* __restrict__ x, const TD* __restrict__ de
 template <typename TA, typename TD, int NV>
 __global__ __launch_bounds__(256) void postnorm_regs_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_delta,
                                                             long delta_stride, float alpha, const float* __restrict__ gain,
-                                                            float eps, TA* __restrict__ act, int H) {
+                                                            int gain_n, float eps, TA* __restrict__ act, int H) {
     __shared__ float red[16];
     const long r = blockIdx.x;
     float* xr = x + r * H;
@@ -74,13 +75,15 @@ __global__ __launch_bounds__(256) void postnorm_regs_kernel(float* __restrict__ 
         }
     }
     ss = block_sum(ss, red);
-    const float f = rsqrtf(ss / (float)H + eps) * gain[0];
+    const float f = rsqrtf(ss / (float)H + eps) * (gain_n == 1 ? gain[0] : 1.f);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int c = (threadIdx.x + i * blockDim.x) * 4;
         if (c < H) {
+            float gv[4] = {1.f, 1.f, 1.f, 1.f};
+            if (gain_n != 1) Vec4<float>::load(gain + c, gv);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) z[i][k] *= f;
+            for (int k = 0; k < 4; ++k) z[i][k] = gain_n == 1 ? z[i][k] * f : z[i][k] * f * gv[k];
             Vec4<float>::store(xr + c, z[i]);
             if (act) Vec4<TA>::store(act + r * H + c, z[i]);
         }
@@ -89,9 +92,10 @@ __global__ __launch_bounds__(256) void postnorm_regs_kernel(float* __restrict__ 
 
 // dt_d: element type of delta; dt_a: of the copy (act may be null: no copy)
 extern "C" int qe_postnorm(float* x, const void* delta, int n_delta, int dt_d, float alpha, const float* gain,
-                           float eps, void* act, int dt_a, int T, int H, hipStream_t stream) {
+                           int gain_n, float eps, void* act, int dt_a, int T, int H, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && H > 0, "postnorm: bad sizes T=%d H=%d", T, H);
     QE_REQUIRE(!delta || n_delta >= 1, "postnorm: %d delta tensors", n_delta);
+    QE_REQUIRE(gain_n == 1 || gain_n == H, "postnorm: %d gains for rows of %d", gain_n, H);
     if (T == 0) return 0;
     const long stride = (long)T * H;
     const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
@@ -100,9 +104,9 @@ extern "C" int qe_postnorm(float* x, const void* delta, int n_delta, int dt_d, f
     const int nv = regs ? (H / 4 + rthreads - 1) / rthreads : 0;
 #define QE_PN(TA_, TD_)                                                                                                       \
     do {                                                                                                                      \
-        if (regs && nv <= 2) postnorm_regs_kernel<TA_, TD_, 2><<<T, rthreads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H); \
-        else if (regs) postnorm_regs_kernel<TA_, TD_, 8><<<T, rthreads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H); \
-        else postnorm_kernel<TA_, TD_><<<T, threads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H); \
+        if (regs && nv <= 2) postnorm_regs_kernel<TA_, TD_, 2><<<T, rthreads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, gain_n, eps, (TA_*)act, H); \
+        else if (regs) postnorm_regs_kernel<TA_, TD_, 8><<<T, rthreads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, gain_n, eps, (TA_*)act, H); \
+        else postnorm_kernel<TA_, TD_><<<T, threads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, gain_n, eps, (TA_*)act, H); \
     } while (0)
     const int dd = delta ? dt_d : QE_F32;
     if (dt_a == QE_F32 && dd == QE_F32) QE_PN(float, float);

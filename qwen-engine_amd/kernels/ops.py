@@ -85,7 +85,17 @@ def load_library():
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_argmax_static": [vp, vp, i32, i32, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
-        "qe_postnorm": [vp, vp, i32, i32, f32, vp, f32, vp, i32, i32, i32, vp],
+        "qe_postnorm": [vp, vp, i32, i32, f32, vp, i32, f32, vp, i32, i32, i32, vp],
+        "qe_qkv_norm_store": [vp, i32, vp, vp, i32, f32, i32, i32, f32, vp, vp, i32, vp, vp, i32, vp, vp, vp,
+                              i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_attention_talk": [vp, vp, i64, f32, vp, vp, vp, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32,
+                              f32, i32, i32, vp],
+        "qe_token_shift": [vp, vp, i32, vp, i64, vp, vp, i32, i32, i32, i32, vp],
+        "qe_linear_recurrence": [vp, vp, vp, i64, vp, i64, vp, vp, vp, i32, i32, vp, i64, vp, vp, i32, i32, i32, i32,
+                                 i32, vp],
+        "qe_gated_norm": [vp, vp, vp, i64, i32, i32, f32, f32, vp, i64, i32, i32, i32, i32, vp],
+        "qe_unary": [vp, i32, vp, i32, i64, i32, f32, vp],
+        "qe_scaled_sum": [vp, f32, vp, f32, i32, vp, i64, vp],
         "qe_polynorm": [vp, vp, f32, vp, i32, i32, i32, vp],
         "qe_short_conv": [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
         "qe_latent_kv_store": [vp, vp, f32, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, i32, i32, vp],
@@ -616,7 +626,7 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
               other_tiles: Optional[torch.Tensor] = None, prefill_groups: int = 0,
               max_other_keys: int = 0, prefill_segment_keys: int = -1,
               other_keys_row: Optional[int] = None, shared_keys: Optional[torch.Tensor] = None,
-              keep_first: int = 0, sink: bool = False) -> torch.Tensor:
+              keep_first: int = 0, sink: bool = False, chunk: int = 0) -> torch.Tensor:
     """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
     positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
     positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
@@ -637,6 +647,9 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     (other_keys_row): the kernel then cuts by that row's position.
     Without the lists every row is treated alike.
 
+    ``chunk`` (instead of a window): positions are cut into chunks of that many, counted from the request's
+    start, and a token sees the keys of its own chunk up to itself.
+
     shared_keys (int32, an entry per row of block_table, or None): how many of a request's first keys
     other requests read too.  A hint for the decode kernel's loads; results do not depend on it."""
     lib = load_library()
@@ -656,11 +669,15 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     max_blocks = block_table.shape[1]
     if shared_keys is not None:
         _need(shared_keys, "shared_keys", torch.int32, (block_table.shape[0],), dev)
-    keep_first, sink = int(keep_first) if window else 0, int(bool(sink))
+    if chunk:
+        if window or keep_first or chunk < 0:
+            raise KernelError("attention: chunks go without a window and kept first keys")
+        window = -int(chunk)        # (the kernels take a negative window as the length of a chunk)
+    keep_first, sink = int(keep_first) if window > 0 else 0, int(bool(sink))
     if keep_first < 0:
         raise KernelError("attention: negative keep_first")
-    if keep_first or sink:
-        prefill_segment_keys = 0
+    if keep_first or sink or chunk:
+        prefill_segment_keys = 0    # (no segments of keys: such walks are short)
 
     def generic(tokens):
         n = T if tokens is None else tokens.shape[0]
@@ -862,12 +879,14 @@ def postnorm(x: torch.Tensor, delta: Optional[torch.Tensor], alpha: float, gain:
              act_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
     """x <- gain * z / sqrt(mean(z^2) + eps) with z = alpha * x + delta, on the 32-bit stream x [T, H], in
     place.  delta: None, [T, H] (bfloat16 or float32) or float32 [S, T, H], added in the order of S.  gain:
-    float32 [1].  With ``act_dtype`` bfloat16 a copy of the new x in that type is returned (what the next
+    float32 [1] (one for all coordinates) or [H].  With ``act_dtype`` bfloat16 a copy of the new x in that type is returned (what the next
     products read); with float32 or None, nothing (the stream itself is read)."""
     lib = load_library()
     _need(x, "x", torch.float32, (None, None))
     T, H = x.shape
-    _need(gain, "gain", torch.float32, (1,), x.device)
+    _need(gain, "gain", torch.float32, (None,), x.device)
+    if gain.shape[0] not in (1, H):
+        raise KernelError(f"postnorm: {gain.shape[0]} gains for rows of {H}")
     n_delta, dt_d = 0, F32
     if delta is not None:
         if delta.dim() == 3:
@@ -879,7 +898,7 @@ def postnorm(x: torch.Tensor, delta: Optional[torch.Tensor], alpha: float, gain:
     act = None
     if act_dtype == torch.bfloat16:
         act = torch.empty((T, H), dtype=torch.bfloat16, device=x.device)
-    _check(lib.qe_postnorm(x.data_ptr(), _ptr(delta), n_delta, dt_d, float(alpha), gain.data_ptr(), float(eps),
+    _check(lib.qe_postnorm(x.data_ptr(), _ptr(delta), n_delta, dt_d, float(alpha), gain.data_ptr(), gain.shape[0], float(eps),
                            _ptr(act), BF16 if act is not None else F32, T, H, _stream()), "postnorm")
     return act
 
@@ -1250,3 +1269,218 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
                            _DT[x.dtype], _DT[w_down.dtype], _stream()), "moe_gemm (down)")
     identity(parts, None)
     return parts
+
+
+# ---- queries, keys and values normed over the whole projection or per head; values from keys; blended values --------
+QK_NORM_NONE, QK_NORM_HEAD, QK_NORM_WHOLE = 0, 1, 2
+
+
+def qkv_norm_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, k_dim: int, v_dim: int, cache: torch.Tensor,
+                   slots: Optional[torch.Tensor], qk_norm: int = QK_NORM_NONE, q_weight: Optional[torch.Tensor] = None,
+                   k_weight: Optional[torch.Tensor] = None, qk_eps: float = 0.0, values_from_keys: bool = False,
+                   value_norm_eps: Optional[float] = None, v_first: Optional[torch.Tensor] = None,
+                   v_blend: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
+                   inv_freq: Optional[torch.Tensor] = None, value_rows: bool = False) -> torch.Tensor:
+    """From the projected rows qkv [T, Hq k_dim + Hkv k_dim (+ Hkv v_dim)] to q [T, Hq, Dc] and the cache
+    [pages, 2, Hkv, P, Dc] (zeros beyond a head's own numbers): q and k normed per head (weights [k_dim]) or
+    over the whole projection (weights [Hq k_dim] and [Hkv k_dim]), the values their own projection or the keys
+    as projected (``values_from_keys``), each value head divided by its root mean square (``value_norm_eps``),
+    then either left in ``v_first`` (float32 [T, Hkv v_dim]; ``v_blend`` None) for later layers or blended with
+    it, v <- (1 - v_blend) v + v_blend v_first; the first 2 len(inv_freq) numbers of every q and k head rotated in
+    half-split pairs by positions * inv_freq; k and v written at ``slots`` (page * P + offset; negative: nowhere),
+    value tiles transposed ([Dc][P]) or, with ``value_rows``, as rows ([P][Dc])."""
+    lib = load_library()
+    _need(qkv, "qkv", _ACT, (None, None))
+    T, dev = qkv.shape[0], qkv.device
+    Hq, Hkv, Dk, Dv = int(num_heads), int(num_kv_heads), int(k_dim), int(v_dim)
+    need = Hq * Dk + Hkv * Dk + (0 if values_from_keys else Hkv * Dv)
+    if qkv.shape[1] != need:
+        raise KernelError(f"qkv_norm_store: rows of {qkv.shape[1]} numbers, {need} expected")
+    _need(cache, "cache", qkv.dtype, (None, 2, Hkv, None, None), dev)
+    P, Dc = cache.shape[3], cache.shape[4]
+    if qk_norm != QK_NORM_NONE:
+        n = (Hq * Dk, Hkv * Dk) if qk_norm == QK_NORM_WHOLE else (Dk, Dk)
+        _need(q_weight, "q_weight", torch.float32, (n[0],), dev)
+        _need(k_weight, "k_weight", torch.float32, (n[1],), dev)
+    if slots is not None:
+        _need(slots, "slots", torch.int32, (T,), dev)
+    if v_first is not None:
+        _need(v_first, "v_first", torch.float32, (T, Hkv * Dv), dev)
+        if v_blend is not None:
+            _need(v_blend, "v_blend", torch.float32, (1,), dev)
+    elif v_blend is not None:
+        raise KernelError("qkv_norm_store: a blend without the values to blend with")
+    rot = 0
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (None,), dev)
+        _need(positions, "positions", torch.int32, (T,), dev)
+        rot = 2 * inv_freq.shape[0]
+    q = torch.empty((T, Hq, Dc), dtype=qkv.dtype, device=dev)
+    _check(lib.qe_qkv_norm_store(qkv.data_ptr(), qkv.shape[1], _ptr(q_weight), _ptr(k_weight), int(qk_norm), float(qk_eps),
+                                 int(bool(values_from_keys)), int(value_norm_eps is not None),
+                                 float(value_norm_eps or 0.0), _ptr(v_blend), _ptr(v_first),
+                                 int(v_first is not None and v_blend is None), _ptr(positions), _ptr(inv_freq), rot,
+                                 _ptr(slots), q.data_ptr(), cache.data_ptr(), T, Hq, Hkv, Dk, Dv, Dc, P,
+                                 int(bool(value_rows)), _DT[qkv.dtype], _stream()), "qkv_norm_store")
+    return q
+
+
+def attention_talk(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
+                   block_table: torch.Tensor, scale: float, k_dim: int, v_dim: int, window: int = 0, chunk: int = 0,
+                   bias: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
+                   out: Optional[torch.Tensor] = None, out_scale: float = 1.0,
+                   tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention whose scores get a bias by distance (``bias`` float32 [rows, Hq]: row min(i - j, rows - 1)) and are
+    then mixed across heads (``talk`` float32 [Hq, Hq]: s'_h = sum_g talk[h, g] s_g) before the softmax.  q
+    [T, Hq, Dc]; cache [pages, 2, Hkv, P, Dc] with keys and values both as rows; a head's keys have k_dim numbers,
+    its values v_dim.  ``window`` / ``chunk`` as for attention().  out [T, Hq * v_dim] (may be a slice of columns
+    of a wider tensor), multiplied by out_scale."""
+    lib = load_library()
+    _need(q, "q", _ACT, (None, None, None))
+    T, Hq, Dc = q.shape
+    dev = q.device
+    _need(cache, "cache", q.dtype, (None, 2, None, None, Dc), dev)
+    Hkv, P = cache.shape[2], cache.shape[3]
+    _need(positions, "positions", torch.int32, (T,), dev)
+    _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
+    _need(block_table, "block_table", torch.int32, (None, None), dev)
+    if chunk:
+        if window or chunk < 0:
+            raise KernelError("attention_talk: chunks go without a window")
+        window = -int(chunk)
+    rows = 0
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (None, Hq), dev)
+        rows = bias.shape[0]
+    if talk is not None:
+        _need(talk, "talk", torch.float32, (Hq, Hq), dev)
+    n = Hq * int(v_dim)
+    if out is None:
+        out = torch.empty((T, n), dtype=q.dtype, device=dev)
+    if out.dtype != q.dtype or out.dim() != 2 or out.shape != (T, n) or out.stride(1) != 1 or out.device != dev:
+        raise KernelError(f"attention_talk: out is {tuple(out.shape)} {out.dtype}, expected {(T, n)} {q.dtype}")
+    n_tok = T
+    if tokens is not None:
+        _need(tokens, "tokens", torch.int32, (None,), dev)
+        n_tok = tokens.shape[0]
+    _check(lib.qe_attention_talk(q.data_ptr(), out.data_ptr(), out.stride(0) if T > 1 else n, float(out_scale),
+                                 cache.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
+                                 block_table.shape[1], _ptr(tokens), n_tok, _ptr(bias), rows, _ptr(talk), Hq, Hkv,
+                                 int(k_dim), int(v_dim), Dc, P, float(scale), int(window), _DT[q.dtype], _stream()),
+           "attention_talk")
+    return out
+
+
+# ---- mixers with a matrix per head as their state -----------------------------------------------------------------------
+def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, tok_seq: torch.Tensor,
+                single_rows: bool = False) -> torch.Tensor:
+    """y[s] = x + (x' - x) * mu[s], x' the row of the token before in the same request (rows of a request are
+    consecutive; tok_seq names its state row): x [T, W], mu float32 [n, W] -> [n, T, W].  What lies before a request's
+    rows in this step is state[tok_seq[t], :W] (float32; zeros for a new request), which then takes the request's
+    last row.  ``single_rows``: no two rows belong to one request (one launch instead of two)."""
+    lib = load_library()
+    _need(x, "x", _ACT, (None, None))
+    T, W = x.shape
+    _need(mu, "mu", torch.float32, (None, W), x.device)
+    _need(tok_seq, "tok_seq", torch.int32, (T,), x.device)
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < W or state.stride(1) != 1:
+        raise KernelError("token_shift: the state is float32 [slots, >= W]")
+    y = torch.empty((mu.shape[0], T, W), dtype=x.dtype, device=x.device)
+    _check(lib.qe_token_shift(x.data_ptr(), mu.data_ptr(), mu.shape[0], state.data_ptr(), state.stride(0),
+                              tok_seq.data_ptr(), y.data_ptr(), T, W, int(bool(single_rows)), _DT[x.dtype], _stream()),
+           "token_shift")
+    return y
+
+
+def _rows_view(t: torch.Tensor, name: str, n: int, T: int):
+    if t.dim() != 2 or t.shape != (T, n) or t.stride(1) != 1:
+        raise KernelError(f"{name} is {tuple(t.shape)} with strides {t.stride()}, expected rows of {n} numbers")
+    return t.stride(0) if T > 1 else n
+
+
+def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, tok_seq: torch.Tensor,
+                      heads: int, decay: Optional[torch.Tensor] = None, decay_x: Optional[torch.Tensor] = None,
+                      decay_bias: Optional[torch.Tensor] = None, bonus: Optional[torch.Tensor] = None,
+                      silu: bool = False) -> torch.Tensor:
+    """Per head, with a 32-bit state S [D][Dv] per request (state[tok_seq[t]], float32 [slots, >= H D Dv]):
+    with ``decay`` (float32 [H]):  S <- decay_h S + k_t v_t^T, o_t = S^T q_t;
+    with ``decay_x`` float32 [T, H D], ``decay_bias`` and ``bonus`` (float32 [H D]):  o_t = (S + diag(bonus) k_t v_t^T)^T q_t,
+    then S <- diag(w_t) S + k_t v_t^T with w_t = exp(-exp(decay_x_t + decay_bias)).
+    q, k [T, H D], v [T, H Dv] (column slices of one wider tensor are taken as they are, all with one row stride);
+    ``silu``: the three pass silu first.  Returns o float32 [T, H, Dv]."""
+    lib = load_library()
+    T, dev, H = q.shape[0], q.device, int(heads)
+    if q.dtype not in _ACT or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise KernelError("linear_recurrence: q, k and v of one element type")
+    D, Dv = q.shape[1] // H, v.shape[1] // H
+    sq, sk, sv = _rows_view(q, "q", H * D, T), _rows_view(k, "k", H * D, T), _rows_view(v, "v", H * Dv, T)
+    if T > 1 and not sq == sk == sv:
+        raise KernelError("linear_recurrence: q, k and v with different row strides")
+    _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] < H * D * Dv or state.stride(1) != 1:
+        raise KernelError("linear_recurrence: the state is float32 [slots, >= H D Dv]")
+    mode, sw = 0, 0
+    if decay is not None:
+        _need(decay, "decay", torch.float32, (H,), dev)
+    else:
+        mode = 1
+        if decay_x is None or decay_x.dtype != torch.float32:
+            raise KernelError("linear_recurrence: no decays")
+        sw = _rows_view(decay_x, "decay_x", H * D, T)
+        _need(decay_bias, "decay_bias", torch.float32, (H * D,), dev)
+        _need(bonus, "bonus", torch.float32, (H * D,), dev)
+    out = torch.empty((T, H, Dv), dtype=torch.float32, device=dev)
+    _check(lib.qe_linear_recurrence(q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, _ptr(decay_x), sw, _ptr(decay_bias),
+                                    _ptr(bonus), _ptr(decay), mode, int(bool(silu)), state.data_ptr(), state.stride(0),
+                                    tok_seq.data_ptr(), out.data_ptr(), T, H, D, Dv, _DT[q.dtype], _stream()),
+           "linear_recurrence")
+    return out
+
+
+GATE_NONE, GATE_SILU, GATE_SIGMOID = 0, 1, 2
+
+
+def gated_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, groups: int, out_dtype: torch.dtype,
+               gate: Optional[torch.Tensor] = None, gate_act: int = GATE_NONE, scale: float = 1.0,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = o / rms(o) * weight * act(gate) * scale per row of o (float32 [T, N]), the root mean square taken over
+    each of ``groups`` equal pieces of the row; gate [T, N] (may be a slice of columns), act silu or sigmoid."""
+    lib = load_library()
+    _need(o, "o", torch.float32, (None, None))
+    T, N = o.shape
+    _need(weight, "weight", torch.float32, (N,), o.device)
+    sg, dg = 0, F32
+    if gate is not None:
+        sg, dg = _rows_view(gate, "gate", N, T), _DT[gate.dtype]
+    if out is None:
+        out = torch.empty((T, N), dtype=out_dtype, device=o.device)
+    so = _rows_view(out, "out", N, T)
+    _check(lib.qe_gated_norm(o.data_ptr(), weight.data_ptr(), _ptr(gate), sg, dg, int(gate_act), float(eps), float(scale),
+                             out.data_ptr(), so, _DT[out.dtype], T, N, int(groups), _stream()), "gated_norm")
+    return out
+
+
+UNARY_GELU, UNARY_TANH, UNARY_SOFTCAP = 0, 1, 2
+
+
+def unary(z: torch.Tensor, kind: int, out_dtype: Optional[torch.dtype] = None, cap: float = 0.0,
+          inplace: bool = False) -> torch.Tensor:
+    """Element by element in 32-bit: the exact gelu 0.5 z (1 + erf(z / sqrt 2)), tanh, or cap * tanh(z / cap)."""
+    lib = load_library()
+    if not z.is_contiguous() or z.dtype not in _ACT:
+        raise KernelError("unary: a contiguous float32 or bfloat16 tensor")
+    y = z if inplace else torch.empty(z.shape, dtype=out_dtype or z.dtype, device=z.device)
+    _check(lib.qe_unary(z.data_ptr(), _DT[z.dtype], y.data_ptr(), _DT[y.dtype], z.numel(), int(kind), float(cap),
+                        _stream()), "unary")
+    return y
+
+
+def scaled_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float) -> torch.Tensor:
+    """sa * a + sb * b in 32-bit, float32."""
+    lib = load_library()
+    if a.shape != b.shape or a.dtype != b.dtype or a.dtype not in _ACT or not a.is_contiguous() or not b.is_contiguous():
+        raise KernelError("scaled_sum: two contiguous tensors of one shape and type")
+    y = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+    _check(lib.qe_scaled_sum(a.data_ptr(), float(sa), b.data_ptr(), float(sb), _DT[a.dtype], y.data_ptr(), a.numel(),
+                             _stream()), "scaled_sum")
+    return y

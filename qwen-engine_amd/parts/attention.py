@@ -408,5 +408,173 @@ class ConvAttention(PagedAttention):
         return self._project_out(o)
 
 
+def distance_bias_rows(table: torch.Tensor, far: float) -> torch.Tensor:
+    """A learned bias by distance as one row per distance: ``table`` [B, heads] holds a row each for the distances
+    below B // 2 and logarithmic steps up to ``far`` for the rest; distance n reads row n for n < B // 2, else
+    min(B - 1, B // 2 + floor(log(n / (B // 2)) / log(far / (B // 2)) * (B - B // 2))).  Returns float32
+    [ceil(far) + 1, heads]: row n for distance n, the last row for every distance beyond (it is the table's last).
+    The rows are looked up in 64-bit on the host, once."""
+    import math
+    B = table.shape[0]
+    half = B // 2
+    if half < 1 or not far > half:
+        raise ValueError(f"a distance bias of {B} rows up to {far}")
+    rows = []
+    for n in range(int(math.ceil(far)) + 1):
+        if n < half:
+            rows.append(n)
+        else:
+            rows.append(min(B - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (B - half)))))
+    rows[-1] = B - 1
+    return table.float()[torch.tensor(rows)].contiguous()
+
+
+class ChunkAttention(PagedAttention):
+    """Grouped-query attention inside chunks of positions (``ChunkAttentionSpec``): one product for q | k (| v) with
+    the biases; one kernel that norms q and k (per head or over the whole projection), takes the values from their
+    projection or from the keys, norms and blends them, rotates q and k and writes q and the cache; then either the
+    attention kernels of PagedAttention with the chunk as their mask (keys and values of different sizes share the
+    cache under one head size, ``common_head_dim``), or, with a bias by distance or talking heads, the kernel
+    that handles all heads of a token together; then the output projection, whose result stays 32-bit.
+    The values that a layer leaves for later layers of the step travel in ``ctx.memo``."""
+    takes_stream = False
+    graph_safe = True        # every launch's grid follows the rows alone
+
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.hq, self.hkv = int(spec.num_heads), int(spec.num_kv_heads)
+        self.dk, self.dv = int(spec.head_dim), int(spec.v_head_dim)
+        if self.hq % self.hkv:
+            raise ValueError(f"{self.hq} query heads are no multiple of {self.hkv} key/value heads")
+        if spec.values_from_keys and self.dk != self.dv:
+            raise ValueError("values that are the keys have the keys' size")
+        if spec.qk_norm not in (None, "head", "whole"):
+            raise ValueError(f"unknown q/k norm {spec.qk_norm!r}")
+        if spec.value_blend not in (None, "source", "blend"):
+            raise ValueError(f"unknown value blend {spec.value_blend!r}")
+        self.talks = self._talks(spec)
+        self.d = self._cache_head_dim(spec)
+        self.scale = float(spec.scale)
+        self.chunk = int(spec.chunk) if spec.chunk else 0
+        self.window = 0
+        self.position = build_part(spec.position, hidden_size) if spec.position is not None else None
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = None
+        self.blend = self.dist_bias = self.talk = None
+
+    @staticmethod
+    def _talks(spec) -> bool:
+        return bool(spec.distance_bias_rows) or bool(spec.talking_heads)
+
+    @staticmethod
+    def _cache_head_dim(spec) -> int:
+        if ChunkAttention._talks(spec):
+            return (max(int(spec.head_dim), int(spec.v_head_dim)) + 3) // 4 * 4
+        return common_head_dim(spec.head_dim, spec.v_head_dim)
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        nq, nk, nv, no = spec.names
+        rows = {nq: spec.num_heads * spec.head_dim, nk: spec.num_kv_heads * spec.head_dim}
+        if not spec.values_from_keys:
+            rows[nv] = spec.num_kv_heads * spec.v_head_dim
+        t = {}
+        for name, n in rows.items():
+            t[name] = TensorInfo((n, hidden))
+            if spec.bias:
+                t[name + spec.bias_suffix] = TensorInfo((n,), "zeros", "vector")
+        if spec.qk_norm is not None:
+            for name in (nq, nk):
+                t[name + spec.norm_suffix] = TensorInfo((rows[name] if spec.qk_norm == "whole" else spec.head_dim,),
+                                                        "ones", "vector")
+        if spec.value_blend is not None:
+            t[spec.blend_name] = TensorInfo((), "zeros", "vector")
+        if spec.distance_bias_rows:
+            t[spec.distance_bias_name] = TensorInfo((int(spec.distance_bias_rows), spec.num_heads), "normal", "vector")
+        if spec.talking_heads:
+            t[spec.talk_name] = TensorInfo((spec.num_heads, spec.num_heads), "normal", "vector")
+        t[no] = TensorInfo((hidden, spec.num_heads * spec.v_head_dim))
+        if spec.bias:
+            t[no + spec.bias_suffix] = TensorInfo((hidden,), "zeros", "vector")
+        return t
+
+    @staticmethod
+    def cache_need(spec) -> Optional[KVNeed]:
+        # (every key stays held: a chunk's first keys are read until the chunk ends)
+        return KVNeed(num_kv_heads=spec.num_kv_heads, head_dim=ChunkAttention._cache_head_dim(spec), window=None)
+
+    @staticmethod
+    def state_need(spec, hidden: int):
+        return None
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        s = self.spec
+        nq, nk, nv, no = s.names
+        proj = [nq, nk] if s.values_from_keys else [nq, nk, nv]
+        mats = [tensors[n] for n in proj]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        self.w_qkv = rt.place_matrix(torch.cat(mats, dim=0))
+        if s.bias:
+            self.b_qkv = rt.place_vector(torch.cat([tensors[n + s.bias_suffix].float() for n in proj]))
+            self.b_o = rt.place_vector(tensors[no + s.bias_suffix])
+        if s.qk_norm is not None:
+            self.q_norm = rt.place_vector(tensors[nq + s.norm_suffix])
+            self.k_norm = rt.place_vector(tensors[nk + s.norm_suffix])
+        if s.value_blend == "blend":
+            self.blend = rt.place_vector(tensors[s.blend_name].reshape(1))
+        if s.distance_bias_rows:
+            self.dist_bias = rt.place_vector(distance_bias_rows(tensors[s.distance_bias_name], float(s.distance_bias_far)))
+        if s.talking_heads:
+            self.talk = rt.place_vector(tensors[s.talk_name])
+        w_o = tensors[no]
+        if self.talks:               # (that kernel writes a head's own values only)
+            self.w_o = rt.place_matrix(w_o)
+        else:                        # heads of the common size: zero columns beyond a value head's own numbers
+            padded = torch.zeros((self.hidden, self.hq, self.d), dtype=w_o.dtype)
+            padded[:, :, :self.dv] = w_o.view(self.hidden, self.hq, self.dv)
+            self.w_o = rt.place_matrix(padded.view(self.hidden, self.hq * self.d))
+        if self.position is not None:
+            self.position.load({}, rt)
+
+    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
+        """x [T, H] in the activation type.  Returns the mixer's output, float32 [T, H]."""
+        if binding.kv is None:
+            raise RuntimeError("attention was given no cache")
+        s = self.spec
+        T, g, cache = x.shape[0], binding.group, binding.kv
+        qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
+        v_first = None
+        if s.value_blend is not None:
+            key = ("chunk_attention.values", self.hkv * self.dv)
+            if s.value_blend == "source":
+                v_first = ctx.memo[key] = torch.empty((T, self.hkv * self.dv), dtype=torch.float32, device=x.device)
+            else:
+                v_first = ctx.memo.get(key)
+                if v_first is None:
+                    raise RuntimeError("values to blend with: no layer before this one has left any")
+        mode = {None: ops.QK_NORM_NONE, "head": ops.QK_NORM_HEAD, "whole": ops.QK_NORM_WHOLE}[s.qk_norm]
+        q = ops.qkv_norm_store(qkv, self.hq, self.hkv, self.dk, self.dv, cache, ctx.slots[g] if binding.write else None,
+                               qk_norm=mode, q_weight=self.q_norm, k_weight=self.k_norm, qk_eps=float(s.qk_norm_eps),
+                               values_from_keys=bool(s.values_from_keys), value_norm_eps=s.value_norm_eps,
+                               v_first=v_first, v_blend=self.blend if s.value_blend == "blend" else None,
+                               positions=ctx.positions,
+                               inv_freq=self.position.inv_freq() if self.position is not None else None,
+                               value_rows=self.talks)
+        if self.talks:
+            o = ops.attention_talk(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.dk,
+                                   self.dv, chunk=self.chunk, bias=self.dist_bias, talk=self.talk)
+        else:
+            ex = self._extras(ctx)
+            o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, 0,
+                              dec_tokens=ex["dec_tokens"], max_dec_position=ex["max_dec_position"],
+                              other_tokens=ex["other_tokens"],
+                              other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None,
+                              max_other_keys=ex.get("max_other_keys", 0), other_keys_row=ex.get("other_keys_row"),
+                              shared_keys=ctx.shared_keys, chunk=self.chunk).view(T, self.hq * self.d)
+        return ops.gemm(o, self.w_o, self.b_o, out_dtype=torch.float32)
+
+
 register_part("paged_attention", PagedAttention)
 register_part("conv_attention", ConvAttention)
+register_part("chunk_attention", ChunkAttention)

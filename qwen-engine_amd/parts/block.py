@@ -115,6 +115,9 @@ class PostNormBlock:
     def graph_safe_with_state(self) -> bool:
         return all(getattr(p, "graph_safe", False) is True for p in (self.mixer, self.conv) if p is not None)
 
+    # the stream's copy in the activation type that the block's last norm made, for the block after it
+    _COPY = "postnorm_block.copy"
+
     @staticmethod
     def _named(spec):
         """(checkpoint name, part spec, optional) of the block's parts."""
@@ -134,9 +137,9 @@ class PostNormBlock:
         kv = cls.cache_need(spec.mixer) if hasattr(cls, "cache_need") else None
         state = part_class(spec.conv.kind).state_need(spec.conv, hidden) if spec.conv is not None else None
         mixer_state = cls.state_need(spec.mixer, hidden) if hasattr(cls, "state_need") else None
-        if mixer_state is not None:
+        if mixer_state is not None and state is not None:
             raise ValueError("a post-norm block's state slot belongs to its convolution: the mixer cannot ask for one too")
-        return [(kv, state)]
+        return [(kv, state if state is not None else mixer_state)]
 
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
@@ -173,17 +176,24 @@ class PostNormBlock:
         if pending is not None:
             ops.residual_add(x, pending)
         binding = bindings[0]
+        kept = ctx.memo.pop(self._COPY, None) if pending is None else None
         if self.conv is not None:
             xin = self.conv.forward(x, ctx, binding.state)
+        elif rt.dtype == torch.float32:
+            xin = x
+        elif kept is not None and kept[0] is x:
+            xin = kept[1]              # (the norm of the block before left its copy: nothing is converted again)
         else:
-            xin = x if rt.dtype == torch.float32 else x.to(rt.dtype)
+            xin = x.to(rt.dtype)
         y = self.mixer.forward(xin, ctx, binding)
         xa = self.mixer_norm.after_sum(x, y, self.alpha, rt)
         if self.ffn is not None:
             y = self.ffn.forward(x if xa is None else xa, ctx)
-            self.ffn_norm.after_sum(x, y, self.alpha, rt)
+            xa = self.ffn_norm.after_sum(x, y, self.alpha, rt)
         elif self.has_ffn_norm:
-            self.ffn_norm.after_sum(x, None, self.alpha, rt)
+            xa = self.ffn_norm.after_sum(x, None, self.alpha, rt)
+        if xa is not None:
+            ctx.memo[self._COPY] = (x, xa)
         return None
 
 

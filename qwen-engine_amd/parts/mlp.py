@@ -64,4 +64,31 @@ class SwiGLU:
         return ops.gemm(a, self.w_down)
 
 
+class GeluMLP:
+    """down(gelu(up x)), the exact gelu; the up product's result stays 32-bit until the activation has been applied
+    (one rounding), and the output is handed on in 32-bit for the residual sum."""
+
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.inter = int(spec.intermediate_size)
+        self.w_up = self.w_down = None
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        up, down = spec.names
+        return {up: TensorInfo((spec.intermediate_size, hidden)), down: TensorInfo((hidden, spec.intermediate_size))}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        up, down = self.spec.names
+        self.w_up = rt.place_matrix(tensors[up])
+        self.w_down = rt.place_matrix(tensors[down])
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        z = ops.gemm(x, self.w_up, out_dtype=torch.float32)
+        a = ops.unary(z, ops.UNARY_GELU, out_dtype=ctx.rt.dtype)
+        return ops.gemm(a, self.w_down, out_dtype=torch.float32)
+
+
 register_part("swiglu", SwiGLU)
+register_part("gelu_mlp", GeluMLP)

@@ -32,6 +32,11 @@ class RMSNorm:
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.rmsnorm(h, self.weight, self.eps, rt.dtype, delta=delta, rows=rows)
 
+    def after_sum(self, x: torch.Tensor, delta: Optional[torch.Tensor], alpha: float, rt: Runtime):
+        """The norm of a post-norm block: x <- w * z / rms(z) with z = alpha * x + delta, on the 32-bit stream in
+        place; returns the new x in the activation type where that is not 32-bit."""
+        return ops.postnorm(x, delta, alpha, self.weight, self.eps, rt.dtype)
+
 
 class ScalarRMSNorm:
     """RMS norm with one gain for all coordinates (a tensor of no dimensions, named as the part itself).
@@ -89,7 +94,27 @@ class StreamScale:
         ops.scale_(h, self.scale)
 
 
+class LogitSoftcap:
+    """logits <- cap * tanh(logits / cap), in place on the 32-bit logits."""
+
+    def __init__(self, spec, hidden_size: int = 0):
+        self.cap = float(spec.cap)
+        if not self.cap > 0:
+            raise ValueError(f"a soft cap of {self.cap}")
+
+    @staticmethod
+    def expected_tensors(spec, hidden_size: int) -> Dict[str, TensorInfo]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        pass
+
+    def forward(self, logits: torch.Tensor, ctx) -> torch.Tensor:
+        return ops.unary(logits, ops.UNARY_SOFTCAP, cap=self.cap, inplace=True)
+
+
 register_part("rmsnorm", RMSNorm)
+register_part("logit_softcap", LogitSoftcap)
 register_part("rmsnorm_bare", BareRMSNorm)
 register_part("stream_scale", StreamScale)
 register_part("rmsnorm_scalar", ScalarRMSNorm)
