@@ -35,8 +35,9 @@ Other sizes and workloads (not what the default line reports):
                             recorded graph of repetitions over weights that do not fit the caches, and its rate
                             against the nominal and the measured peaks (the counterpart of the reference's
                             per-operator benchmarks, src/layers/ops/linear.py:204-249)
-  --design zarorax|nufavik  another design beside the closest Qwen3 model of equal sizes (width, layers, heads, and a
-                            feed-forward as wide as the experts a token uses): prefill (one prompt of --prefill-tokens
+  --design zarorax|nufavik|potatar
+                            another design beside the closest Qwen3 model of equal sizes (width, layers, heads, and a
+                            feed-forward as wide as the experts a token uses, or of as many weights): prefill (one prompt of --prefill-tokens
                             in one step) and decode (batch 1 and --batch at --context) of both, at the sizes of
                             --design-sizes (small, medium); one JSON line of its own.  The default line is unchanged.
   --warmup-passes N         both: untimed passes over the workload with other tokens before the timed
@@ -94,7 +95,7 @@ def parse():
                     help="run steps of single new tokens beside a prompt portion as they come, not from a recorded graph")
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
     ap.add_argument("--kernels", action="store_true", help="time each kernel of a layer alone over a range of rows")
-    ap.add_argument("--design", default=None, choices=["zarorax", "nufavik"],
+    ap.add_argument("--design", default=None, choices=["zarorax", "nufavik", "potatar"],
                     help="measure this design beside the closest Qwen3 model of equal sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes (small, medium), with commas")
     ap.add_argument("--warmup-passes", type=int, default=2,
@@ -385,6 +386,38 @@ def nufavik_config(z, layers, vocab):
             "layers": [layer] * layers}
 
 
+# Layer sizes for --design potatar: (width, query heads, key/value heads, key and value size, rotated numbers, chunk,
+# rows of the bias by distance and its farthest distance, heads and sizes of the two recurrences, rank of the decay, ff)
+POTATAR_SIZES = {
+    "small": dict(width=1024, heads=16, kv_heads=4, dim=64, vdim=64, rot_dims=32, chunk=1024, bias_rows=32, bias_max=1024,
+                  rec_heads=16, rec_dim=64, decay_rank=64, ff=4096),
+    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, rot_dims=64, chunk=1024, bias_rows=32, bias_max=1024,
+                   rec_heads=16, rec_dim=128, decay_rank=64, ff=8192),
+}
+
+
+def potatar_config(z, layers, vocab):
+    """Attention, the two mixers side by side, attention, the recurrence over shifted tokens (without a feed-forward),
+    in turn."""
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"],
+                     "scale": z["dim"] ** -0.5, "mask": {"size": z["chunk"]}, "rot": {"base": 10000.0, "dims": z["rot_dims"]},
+                     "v_mix": True}}
+    h = z["rec_heads"]
+    side = {"type": "parallel", "mlp": mlp,
+            "mixer": {"left": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                               "scale": z["dim"] ** -0.5, "mask": {"size": z["chunk"]}, "bias_max": z["bias_max"],
+                               "bias_rows": z["bias_rows"]},
+                      "right": {"heads": h, "dim": z["rec_dim"], "vdim": z["rec_dim"],
+                                "decay": [1.0 - 2.0 ** (-3 - 5 * i / max(1, h - 1)) for i in range(h)]},
+                      "left_scale": 1.0, "right_scale": 1.0}}
+    wkv = {"type": "wkv", "mlp": None, "mixer": {"heads": h, "dim": z["rec_dim"], "decay_rank": z["decay_rank"]}}
+    order = [att, side, att, wkv]
+    return {"architecture": "Potatar", "vocab": vocab, "width": z["width"], "postln_alpha": 2.0, "logit_softcap": 30.0,
+            "norm": {"eps": 1e-5}, "layers": [order[i % 4] for i in range(layers)]}
+
+
 def design_compare(args) -> int:
     """Prefill and decode of another design beside the Qwen3 model of equal sizes, through the same step
     function.  A "step" is one decode step; the line's value is the design's decode rate at --batch, first size."""
@@ -453,7 +486,12 @@ def design_compare(args) -> int:
     design = args.design
     title = design.capitalize()
     for name in [n for n in args.design_sizes.split(",") if n]:
-        if design == "nufavik":
+        if design == "potatar":
+            z = POTATAR_SIZES[name]
+            zcfg = config_from_dict(potatar_config(z, layers, V))
+            kv_heads, head_dim = z["kv_heads"], z["dim"]
+            z = dict(z, top=1, expert_ff=z["ff"] * 2 // 3 // 256 * 256)      # (three matrices of as many weights as the two)
+        elif design == "nufavik":
             z = NUFAVIK_SIZES[name]
             zcfg = config_from_dict(nufavik_config(z, layers, V))
             kv_heads, head_dim = z["kv_heads"], max(z["dim"], z["vdim"])
