@@ -56,7 +56,7 @@ PB = {"architecture": "Potatar", "vocab": 300, "width": 128, "norm": {"eps": 1e-
           parallel(4, 4, 64, 40, 0.12, 100.5, 2, 64, 128, (0.8, 0.99), 1.5, 0.5, ff(96)),
           attention(8, 2, 64, 64, 40, 32, 0.11, True, 500000.0, ff(64)),
           wkv(2, 64, None),
-          attention(2, 2, 128, 32, 100, 64, 0.08, True, 10000.0, ff(128)),
+          attention(2, 2, 128, 64, 100, 64, 0.08, True, 10000.0, ff(128)),
       ]}
 SHAPE_SIZES["B"] = {0: 14, 2: 24}
 # C: values that are 1 or equal: alpha 1, one head, sixteen query heads on one key/value head, chunks of one position
