@@ -3,165 +3,360 @@
 //   s'_h      = sum_g talk[h][g] * s_g                                         (the heads' scores mixed)
 //   o_h(i)    = sum_j softmax_j(s'_h(i, .)) v(j)
 // Both the bias and the mixing are optional.  Because a head's weights depend on every head's scores against a
-// key, one block handles all heads of one token: for 64 keys at a time it forms all scores, mixes them, takes
-// the tile into each head's running softmax and adds the tile's values.  Keys are walked from the first key
-// the token sees (first_seen_key: all, a window of the last keys, or the token's own chunk), so the order of
-// the sums depends on the position alone: not on how the request was cut into steps, nor on the batch.  All
-// arithmetic in 32-bit.
+// key, one block handles all heads of one token.  Keys are walked 64 at a time from the first key the token sees
+// (first_seen_key: all, a window of the last keys, or the token's own chunk).  For a tile of 64 keys the block
+//   - brings the key rows of as many key/value heads as fit a staging buffer into shared memory (contiguous loads,
+//     converted to 32-bit, rows padded so that a lane per key reads its row without bank conflicts), and every
+//     wave takes query heads in turn, a lane per key, for the dot products;
+//   - mixes the heads' scores and takes the tile into each head's running softmax (a wave per head);
+//   - brings the value rows into the same buffer and adds the tile's values, a thread per output number.
+// With KS > 1 the tiles of a token are dealt to KS blocks in turn; each leaves its maxima, sums and accumulators in a
+// workspace and attention_talk_merge_kernel weighs and adds them in the order of the splits.  The order of the sums
+// depends on the position and KS alone: not on how the request was cut into steps.  All arithmetic in 32-bit.
 //
-// cache of one layer: [page][2 (k, v)][Hkv][P][Dc], keys and values both as rows.
+// cache of one layer: [page][2 (k, v)][Hkv][P][Dc], keys and values both as rows, zeros beyond a head's own numbers,
+// Dc a multiple of 4.
 #include "common.h"
 
 #define TALK_THREADS 256
-#define TALK_MAX_ACC 16          // outputs a thread: Hq * Dv <= 256 * 16
+#define TALK_MAX_ACC 4           // groups of four outputs a thread: Hq * ceil(Dv / 4) <= 256 * 4
+#define TALK_MAX_SPLITS 16
 
-template <typename TA>
+// Four consecutive elements as they lie in memory, and as four floats.
+template <typename T> struct Raw4;
+template <> struct Raw4<float> {
+    typedef float4 R;
+    static __device__ __forceinline__ R load(const float* p) { return *(const float4*)p; }
+    static __device__ __forceinline__ R zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+    static __device__ __forceinline__ float4 widen(R r) { return r; }
+};
+template <> struct Raw4<bf16_t> {
+    typedef uint2 R;
+    static __device__ __forceinline__ R load(const bf16_t* p) { return *(const uint2*)p; }
+    static __device__ __forceinline__ R zero() { return make_uint2(0u, 0u); }
+    static __device__ __forceinline__ float4 widen(R r) {
+        return make_float4(bf16_bits_to_float(r.x & 0xffffu), bf16_bits_to_float(r.x >> 16),
+                           bf16_bits_to_float(r.y & 0xffffu), bf16_bits_to_float(r.y >> 16));
+    }
+};
+
+struct TalkLayout {              // offsets into shared memory, in floats (all multiples of 4)
+    int rs_q, ls_k, ls_v, stage, sc, pm, small, total;
+};
+
+__host__ __device__ __forceinline__ TalkLayout talk_layout(int Hq, int Dk, int Dv, int HGk, int HGv) {
+    TalkLayout L;
+    L.rs_q = (Dk + 3) & ~3;
+    L.ls_k = L.rs_q + (((L.rs_q >> 2) & 1) ? 0 : 4);      // an odd number of 16-byte pieces a row
+    L.ls_v = (Dv + 3) & ~3;
+    const int a = HGk * 64 * L.ls_k, b = HGv * 64 * L.ls_v;
+    L.stage = 256 + Hq * L.rs_q;                           // (256 floats = twice 64 offsets of 8 bytes come first)
+    L.sc = L.stage + (a > b ? a : b);
+    L.pm = L.sc + Hq * 64;
+    L.small = L.pm + Hq * 64;
+    L.total = L.small + ((3 * Hq + Hq * Hq + 3) & ~3);
+    return L;
+}
+
+// A stage: the rows of `hg` key/value heads from g0, of one plane, of a tile's 64 keys.  talk_fetch starts the
+// loads of a stage into registers (NV pieces of four numbers a thread; keys that are not seen, offset < 0, become
+// zeros); talk_commit writes them to stage[gl][jj][ls] in 32-bit.  Between the two the block computes on the stage
+// before.
+// item[u]: (row of the stage << 8) | piece of the row, for the thread's u-th piece of a stage; -1: beyond a full stage
+template <int NV>
+__device__ __forceinline__ void talk_items(int (&item)[NV], int hmax, int vec_per_row) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = threadIdx.x + u * TALK_THREADS;
+        item[u] = i < hmax * 64 * vec_per_row ? ((i / vec_per_row) << 8) | (i % vec_per_row) : -1;
+    }
+}
+
+template <typename TA, int NV>
+__device__ __forceinline__ void talk_fetch(typename Raw4<TA>::R (&regs)[NV], const int (&item)[NV],
+                                           const TA* __restrict__ plane, const long* koff, int g0, int hg,
+                                           long head_stride) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        typename Raw4<TA>::R r = Raw4<TA>::zero();
+        const int rr = item[u] >> 8;
+        if (item[u] >= 0 && rr < hg * 64) {
+            const long off = koff[rr & 63];
+            if (off >= 0) r = Raw4<TA>::load(plane + off + (long)(g0 + (rr >> 6)) * head_stride + (item[u] & 255) * 4);
+        }
+        regs[u] = r;
+    }
+}
+
+template <typename TA, int NV>
+__device__ __forceinline__ void talk_commit(const typename Raw4<TA>::R (&regs)[NV], const int (&item)[NV],
+                                            float* stage, int hg, int ls) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int rr = item[u] >> 8;
+        if (item[u] >= 0 && rr < hg * 64)
+            *(float4*)(stage + (long)rr * ls + (item[u] & 255) * 4) = Raw4<TA>::widen(regs[u]);      // (rr = gl * 64 + jj)
+    }
+}
+
+template <typename TA, int NV>
 __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
     const TA* __restrict__ q, TA* __restrict__ out, long out_stride, float out_scale, const TA* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ tokens, const float* __restrict__ bias, int bias_rows,
-    const float* __restrict__ talk, int Hq, int Hkv, int Dk, int Dv, int Dc, int P, float scale, int window) {
-    extern __shared__ float sm[];
-    float* qs = sm;                               // Hq * Dk
-    float* sc = qs + Hq * Dk;                     // Hq * 64 scores
-    float* pm = sc + Hq * 64;                     // Hq * 64 weights
-    float* ml = pm + Hq * 64;                     // Hq * 2 running maximum and sum
-    float* al = ml + Hq * 2;                      // Hq factors of the tile
+    const float* __restrict__ talk, int Hq, int Hkv, int Dk, int Dv, int Dc, int P, float scale, int window,
+    int KS, int HGk, int HGv, float* __restrict__ ws) {
+    extern __shared__ __align__(16) float sm[];
+    const TalkLayout L = talk_layout(Hq, Dk, Dv, HGk, HGv);
+    long* koff = (long*)sm;                       // twice 64 key rows: this tile's and the next one's (-1: not seen)
+    float* qs = sm + 256;                         // Hq rows of rs_q
+    float* stage = sm + L.stage;
+    float* sc = sm + L.sc;                        // Hq * 64 scores
+    float* pm = sm + L.pm;                        // Hq * 64 weights
+    float* ml = sm + L.small;                     // Hq * 2 running maximum and sum
+    float* al = ml + 2 * Hq;                      // Hq factors of the tile
     float* tk = al + Hq;                          // Hq * Hq (if talk)
-    long* voff = (long*)(tk + ((Hq * Hq + 1) & ~1));   // 64 value rows of the tile
     const long t = tokens ? tokens[blockIdx.x] : blockIdx.x;
+    const int split = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int G = Hq / Hkv;
     const int p = positions[t];
     const int lo = first_seen_key(p, window);
     const int* bt = block_table + (long)tok_seq[t] * max_blocks;
-    const long page_stride = 2L * Hkv * P * Dc, plane = (long)Hkv * P * Dc;
+    const long page_stride = 2L * Hkv * P * Dc, plane = (long)Hkv * P * Dc, head_stride = (long)P * Dc;
+    const int n_out = Hq * Dv;
+    const int nK = (Hkv + HGk - 1) / HGk, nS = nK + (Hkv + HGv - 1) / HGv;      // stages of a tile: keys, then values
+    const int vpr_k = L.rs_q >> 2, vpr_v = L.ls_v >> 2;
 
-    for (int i = tid; i < Hq * Dk; i += TALK_THREADS) {
-        const int h = i / Dk, d = i - h * Dk;
-        qs[i] = Elem<TA>::load(q + (t * Hq + h) * Dc + d);
+    for (int i = tid; i < Hq * L.rs_q; i += TALK_THREADS) {
+        const int h = i / L.rs_q, d = i - h * L.rs_q;
+        qs[i] = d < Dk ? Elem<TA>::load(q + (t * Hq + h) * Dc + d) : 0.f;
     }
     if (talk) for (int i = tid; i < Hq * Hq; i += TALK_THREADS) tk[i] = talk[i];
     for (int h = tid; h < Hq; h += TALK_THREADS) { ml[2 * h] = -INFINITY; ml[2 * h + 1] = 0.f; }
-    float acc[TALK_MAX_ACC];
-#pragma unroll
-    for (int i = 0; i < TALK_MAX_ACC; ++i) acc[i] = 0.f;
-    const int n_out = Hq * Dv;
-    __syncthreads();
-
-    for (int j0 = lo; j0 <= p; j0 += 64) {
-        const int j = j0 + lane;
-        const bool seen = j <= p;
-        long koff = 0;
-        if (seen) {
-            const long page = bt[j / P];
-            koff = page * page_stride + (long)(j % P) * Dc;
-        }
-        if (wave == 0) voff[lane] = koff + plane;
-        // ---- scores of the tile: thread (wave, lane) takes heads wave, wave + 4, ... against key j
-        for (int h = wave; h < Hq; h += TALK_THREADS / 64) {
-            float s = 0.f;
-            if (seen) {
-                const TA* kr = cache + koff + (long)(h / G) * P * Dc;
-                const float* qh = qs + h * Dk;
-                float dot = 0.f;
-                if ((Dk & 3) == 0 && (Dc & 3) == 0) {
-                    for (int d = 0; d < Dk; d += 4) {
-                        float kv[4];
-                        Vec4<TA>::load(kr + d, kv);
-                        dot = fmaf(qh[d], kv[0], dot);
-                        dot = fmaf(qh[d + 1], kv[1], dot);
-                        dot = fmaf(qh[d + 2], kv[2], dot);
-                        dot = fmaf(qh[d + 3], kv[3], dot);
-                    }
-                } else {
-                    for (int d = 0; d < Dk; ++d) dot = fmaf(qh[d], Elem<TA>::load(kr + d), dot);
-                }
-                s = dot * scale;
-                if (bias) {
-                    const int n = p - j;
-                    s += bias[(long)(n < bias_rows ? n : bias_rows - 1) * Hq + h];
-                }
-            }
-            sc[h * 64 + lane] = s;
-        }
-        __syncthreads();
-        // ---- the heads' scores mixed, then the tile joins each head's running softmax
-        for (int h = wave; h < Hq; h += TALK_THREADS / 64) {
-            float s;
-            if (talk) {
-                s = 0.f;
-                for (int g = 0; g < Hq; ++g) s = fmaf(tk[h * Hq + g], sc[g * 64 + lane], s);
-            } else {
-                s = sc[h * 64 + lane];
-            }
-            if (!seen) s = -INFINITY;
-            const float m_old = ml[2 * h], l_old = ml[2 * h + 1];
-            const float m_new = fmaxf(m_old, wave_max(s));      // finite: key j0 is always seen
-            const float a = expf(m_old - m_new);                // exp(-inf) = 0 on the first tile
-            const float pj = seen ? expf(s - m_new) : 0.f;
-            const float l_new = l_old * a + wave_sum(pj);
-            pm[h * 64 + lane] = pj;
-            if (lane == 0) { ml[2 * h] = m_new; ml[2 * h + 1] = l_new; al[h] = a; }
-        }
-        __syncthreads();
-        // ---- the tile's values
-        const int cnt = p - j0 + 1 < 64 ? p - j0 + 1 : 64;
-#pragma unroll
-        for (int i = 0; i < TALK_MAX_ACC; ++i) {
-            const int o = tid + i * TALK_THREADS;
-            if (o < n_out) {
-                const int h = o / Dv, d = o - h * Dv;
-                const long hv = (long)(h / G) * P * Dc + d;
-                const float* ph = pm + h * 64;
-                float a = acc[i] * al[h];
-                for (int jj = 0; jj < cnt; ++jj) a = fmaf(ph[jj], Elem<TA>::load(cache + voff[jj] + hv), a);
-                acc[i] = a;
-            }
-        }
-        __syncthreads();
-    }
+    float4 acc[TALK_MAX_ACC];
+    int hd[TALK_MAX_ACC];                          // a group's head and first column
 #pragma unroll
     for (int i = 0; i < TALK_MAX_ACC; ++i) {
+        acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         const int o = tid + i * TALK_THREADS;
-        if (o < n_out) {
-            const int h = o / Dv;
-            Elem<TA>::store(out + t * out_stride + o, acc[i] / ml[2 * h + 1] * out_scale);
+        const int h = o < Hq * vpr_v ? o / vpr_v : Hq;
+        hd[i] = (h << 16) | (h < Hq ? (o - h * vpr_v) * 4 : 0);
+    }
+    typename Raw4<TA>::R regs[NV];
+    int item_k[NV], item_v[NV];
+    talk_items<NV>(item_k, HGk, vpr_k);
+    talk_items<NV>(item_v, HGv, vpr_v);
+
+    int j0 = lo + 64 * split, par = 0;
+    if (j0 <= p) {
+        if (wave == 0) {
+            const int j = j0 + lane;
+            koff[lane] = j <= p ? (long)bt[j / P] * page_stride + (long)(j % P) * Dc : -1L;
+        }
+        __syncthreads();
+        talk_fetch<TA, NV>(regs, item_k, cache, koff, 0, Hkv < HGk ? Hkv : HGk, head_stride);
+    }
+    for (; j0 <= p; j0 += 64 * KS, par ^= 1) {
+        const long* ko = koff + par * 64;
+        long* kn = koff + (par ^ 1) * 64;
+        const int jn = j0 + 64 * KS;
+        const bool more = jn <= p;
+        const int j = j0 + lane;
+        const bool seen = j <= p;
+        if (wave == 0) kn[lane] = jn + lane <= p ? (long)bt[(jn + lane) / P] * page_stride + (long)((jn + lane) % P) * Dc : -1L;
+        for (int s = 0; s < nS; ++s) {
+            const bool is_v = s >= nK;
+            const int g0 = is_v ? (s - nK) * HGv : s * HGk;
+            const int hmax = is_v ? HGv : HGk;
+            const int hg = Hkv - g0 < hmax ? Hkv - g0 : hmax;
+            __syncthreads();                                 // (the stage before has been read)
+            if (is_v) talk_commit<TA, NV>(regs, item_v, stage, hg, L.ls_v);
+            else talk_commit<TA, NV>(regs, item_k, stage, hg, L.ls_k);
+            if (s + 1 < nS) {                                // the next stage's loads fly while this one is computed on
+                const bool nv = s + 1 >= nK;
+                const int n0 = nv ? (s + 1 - nK) * HGv : (s + 1) * HGk;
+                const int nmax = nv ? HGv : HGk;
+                const int nh = Hkv - n0 < nmax ? Hkv - n0 : nmax;
+                if (nv) talk_fetch<TA, NV>(regs, item_v, cache + plane, ko, n0, nh, head_stride);
+                else talk_fetch<TA, NV>(regs, item_k, cache, ko, n0, nh, head_stride);
+            } else if (more) {
+                talk_fetch<TA, NV>(regs, item_k, cache, kn, 0, Hkv < HGk ? Hkv : HGk, head_stride);
+            }
+            __syncthreads();
+            if (!is_v) {
+                // ---- scores: thread (wave, lane) takes heads wave, wave + 4, ... of the staged key heads against key j
+                for (int h = g0 * G + wave; h < (g0 + hg) * G; h += TALK_THREADS / 64) {
+                    const float4* kr = (const float4*)(stage + (long)((h / G - g0) * 64 + lane) * L.ls_k);
+                    const float4* qh = (const float4*)(qs + h * L.rs_q);
+                    float d0 = 0.f, d1 = 0.f;
+                    for (int d = 0; d < vpr_k; ++d) {
+                        const float4 a = qh[d], b = kr[d];
+                        d0 = fmaf(a.x, b.x, d0); d1 = fmaf(a.y, b.y, d1);
+                        d0 = fmaf(a.z, b.z, d0); d1 = fmaf(a.w, b.w, d1);
+                    }
+                    float sv = (d0 + d1) * scale;
+                    if (bias && seen) {
+                        const int n = p - j;
+                        sv += bias[(long)(n < bias_rows ? n : bias_rows - 1) * Hq + h];
+                    }
+                    sc[h * 64 + lane] = sv;
+                }
+                if (s == nK - 1) {
+                    __syncthreads();
+                    // ---- the heads' scores mixed, then the tile joins each head's running softmax
+                    for (int h = wave; h < Hq; h += TALK_THREADS / 64) {
+                        float sv;
+                        if (talk) {
+                            sv = 0.f;
+                            for (int g = 0; g < Hq; ++g) sv = fmaf(tk[h * Hq + g], sc[g * 64 + lane], sv);
+                        } else {
+                            sv = sc[h * 64 + lane];
+                        }
+                        if (!seen) sv = -INFINITY;
+                        const float m_old = ml[2 * h], l_old = ml[2 * h + 1];
+                        const float m_new = fmaxf(m_old, wave_max(sv));     // finite: key j0 is always seen
+                        const float a = expf(m_old - m_new);                // exp(-inf) = 0 on the first tile
+                        const float pj = seen ? expf(sv - m_new) : 0.f;
+                        const float l_new = l_old * a + wave_sum(pj);
+                        pm[h * 64 + lane] = pj;
+                        if (lane == 0) { ml[2 * h] = m_new; ml[2 * h + 1] = l_new; al[h] = a; }
+                    }
+                }
+            } else {
+                // ---- the tile's values (unseen keys: zeros with weight zero)
+#pragma unroll
+                for (int i = 0; i < TALK_MAX_ACC; ++i) {
+                    const int h = hd[i] >> 16, gk = h / G;
+                    if (h < Hq && gk >= g0 && gk < g0 + hg) {
+                        const float* vs = stage + (long)(gk - g0) * 64 * L.ls_v + (hd[i] & 0xffff);
+                        const float4* ph = (const float4*)(pm + h * 64);
+                        const float f = al[h];
+                        float4 a = make_float4(acc[i].x * f, acc[i].y * f, acc[i].z * f, acc[i].w * f);
+#pragma unroll 4
+                        for (int jj = 0; jj < 16; ++jj) {
+                            const float4 w = ph[jj];
+                            const float wa[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const float4 vv = *(const float4*)(vs + (long)(jj * 4 + e) * L.ls_v);
+                                a.x = fmaf(wa[e], vv.x, a.x); a.y = fmaf(wa[e], vv.y, a.y);
+                                a.z = fmaf(wa[e], vv.z, a.z); a.w = fmaf(wa[e], vv.w, a.w);
+                            }
+                        }
+                        acc[i] = a;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (KS == 1) {
+#pragma unroll
+        for (int i = 0; i < TALK_MAX_ACC; ++i) {
+            const int h = hd[i] >> 16, d = hd[i] & 0xffff;
+            if (h < Hq) {
+                const float f = out_scale / ml[2 * h + 1];
+                const float a[4] = {acc[i].x, acc[i].y, acc[i].z, acc[i].w};
+                for (int e = 0; e < 4; ++e)
+                    if (d + e < Dv) Elem<TA>::store(out + t * out_stride + h * Dv + d + e, a[e] * f);
+            }
+        }
+        return;
+    }
+    float* w = ws + ((long)blockIdx.x * KS + split) * (2 * Hq + n_out);
+    for (int i = tid; i < 2 * Hq; i += TALK_THREADS) w[i] = ml[i];
+#pragma unroll
+    for (int i = 0; i < TALK_MAX_ACC; ++i) {
+        const int h = hd[i] >> 16, d = hd[i] & 0xffff;
+        if (h < Hq) {
+            const float a[4] = {acc[i].x, acc[i].y, acc[i].z, acc[i].w};
+            for (int e = 0; e < 4; ++e)
+                if (d + e < Dv) w[2 * Hq + h * Dv + d + e] = a[e];
         }
     }
 }
 
+// grid (tokens): the splits' partial results weighed by exp(m_s - max m) and added in the order of the splits
+template <typename TA>
+__global__ __launch_bounds__(TALK_THREADS) void attention_talk_merge_kernel(
+    const float* __restrict__ ws, TA* __restrict__ out, long out_stride, float out_scale,
+    const int* __restrict__ tokens, int Hq, int Dv, int KS) {
+    const long t = tokens ? tokens[blockIdx.x] : blockIdx.x;
+    const int n_out = Hq * Dv, rec = 2 * Hq + n_out;
+    const float* w = ws + (long)blockIdx.x * KS * rec;
+    for (int o = threadIdx.x; o < n_out; o += TALK_THREADS) {
+        const int h = o / Dv;
+        float m = -INFINITY;
+        for (int s = 0; s < KS; ++s) m = fmaxf(m, w[(long)s * rec + 2 * h]);
+        float l = 0.f, a = 0.f;
+        for (int s = 0; s < KS; ++s) {
+            const float f = expf(w[(long)s * rec + 2 * h] - m);          // (a split without keys: exp(-inf) = 0)
+            l = fmaf(w[(long)s * rec + 2 * h + 1], f, l);
+            a = fmaf(w[(long)s * rec + 2 * Hq + o], f, a);
+        }
+        Elem<TA>::store(out + t * out_stride + o, a / l * out_scale);
+    }
+}
+
+// Into how many blocks a token's key tiles are dealt: none while the tokens alone fill the machine, else a split for
+// every 128 of the most keys a token can see (max_keys: the chunk or window; 0 if unbounded: no split).
+extern "C" int qe_attention_talk_splits(int n_tokens, int max_keys) {
+    if (n_tokens <= 0 || max_keys <= 128) return 1;
+    int ks = (max_keys + 127) / 128;
+    if (ks > TALK_MAX_SPLITS) ks = TALK_MAX_SPLITS;
+    const int room = 1024 / n_tokens;
+    if (ks > room) ks = room;
+    return ks < 1 ? 1 : ks;
+}
+
 // q [T, Hq, Dc] (a head's first Dk numbers are read); out: row t at out + t * out_stride, Hq * Dv numbers,
 // multiplied by out_scale; bias float32 [bias_rows, Hq] or null; talk float32 [Hq, Hq] or null; tokens: null for
-// all T rows, else n_tokens row indices; window as for first_seen_key.
+// all T rows, else n_tokens row indices; window as for first_seen_key; splits from qe_attention_talk_splits with
+// ws of n_tokens * splits * (2 Hq + Hq Dv) floats (null for one split).
 extern "C" int qe_attention_talk(const void* q, void* out, long out_stride, float out_scale, const void* cache,
                                  const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                                  const int* tokens, int n_tokens, const float* bias, int bias_rows, const float* talk,
-                                 int Hq, int Hkv, int Dk, int Dv, int Dc, int P, float scale, int window, int dt_a,
-                                 hipStream_t stream) {
+                                 int Hq, int Hkv, int Dk, int Dv, int Dc, int P, float scale, int window, int splits,
+                                 float* ws, int dt_a, hipStream_t stream) {
     QE_REQUIRE(n_tokens >= 0 && Hq > 0 && Hkv > 0 && Dk > 0 && Dv > 0 && P > 0 && max_blocks > 0, "talking attention: bad sizes");
     QE_REQUIRE(Hq % Hkv == 0, "talking attention: %d query heads are no multiple of %d key/value heads", Hq, Hkv);
-    QE_REQUIRE(Dc >= Dk && Dc >= Dv, "talking attention: heads of %d and %d numbers in a cache of %d", Dk, Dv, Dc);
-    QE_REQUIRE((long)Hq * Dv <= TALK_THREADS * TALK_MAX_ACC, "talking attention: %d heads of %d values are more than %d outputs",
-               Hq, Dv, TALK_THREADS * TALK_MAX_ACC);
+    QE_REQUIRE(Dc % 4 == 0 && Dc >= ((Dk + 3) & ~3) && Dc >= ((Dv + 3) & ~3),
+               "talking attention: heads of %d and %d numbers in a cache of %d (a multiple of 4)", Dk, Dv, Dc);
+    QE_REQUIRE((long)Hq * ((Dv + 3) / 4) <= TALK_THREADS * TALK_MAX_ACC && Hq < 32768,
+               "talking attention: %d heads of %d values are more than %d outputs", Hq, Dv, 4 * TALK_THREADS * TALK_MAX_ACC);
     QE_REQUIRE(!bias || bias_rows > 0, "talking attention: a bias table without rows");
     QE_REQUIRE(out_stride >= (long)Hq * Dv, "talking attention: output rows overlap");
+    QE_REQUIRE(splits >= 1 && splits <= TALK_MAX_SPLITS && (splits == 1 || ws), "talking attention: %d splits", splits);
     if (n_tokens == 0) return 0;
-    const size_t floats = (size_t)Hq * Dk + 2 * (size_t)Hq * 64 + 3 * (size_t)Hq + (((size_t)Hq * Hq + 1) & ~(size_t)1);
-    const size_t shmem = floats * sizeof(float) + 64 * sizeof(long);
+    const TalkLayout L0 = talk_layout(Hq, Dk, Dv, 1, 1);
+    const int vk = L0.rs_q >> 2, vv = L0.ls_v >> 2;
+    QE_REQUIRE(vk <= 64 && vv <= 64, "talking attention: heads of %d and %d numbers (at most 256)", Dk, Dv);
+    const int nv = (vk > 32 || vv > 32) ? 16 : 8;           // pieces a thread holds of a stage: 256 * nv pieces a stage
+    int hgk = 4 * nv / vk, hgv = 4 * nv / vv;
+    hgk = hgk > Hkv ? Hkv : hgk;
+    hgv = hgv > Hkv ? Hkv : hgv;
+    const TalkLayout L = talk_layout(Hq, Dk, Dv, hgk, hgv);
+    const size_t shmem = (size_t)L.total * sizeof(float);
     QE_REQUIRE(shmem <= 150 * 1024, "talking attention: %zu bytes of shared memory", shmem);
-#define QE_TALK(TA_)                                                                                                 \
+    dim3 grid(n_tokens, splits);
+#define QE_TALK2(TA_, NV_)                                                                                           \
     do {                                                                                                             \
         if (shmem > 48 * 1024)                                                                                       \
-            (void)hipFuncSetAttribute((const void*)attention_talk_kernel<TA_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
-        attention_talk_kernel<TA_><<<n_tokens, TALK_THREADS, shmem, stream>>>(                                       \
+            (void)hipFuncSetAttribute((const void*)attention_talk_kernel<TA_, NV_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
+        attention_talk_kernel<TA_, NV_><<<grid, TALK_THREADS, shmem, stream>>>(                                      \
             (const TA_*)q, (TA_*)out, out_stride, out_scale, (const TA_*)cache, positions, tok_seq, block_table,     \
-            max_blocks, tokens, bias, bias_rows, talk, Hq, Hkv, Dk, Dv, Dc, P, scale, window);                       \
+            max_blocks, tokens, bias, bias_rows, talk, Hq, Hkv, Dk, Dv, Dc, P, scale, window, splits, hgk, hgv, ws); \
+        if (splits > 1)                                                                                              \
+            attention_talk_merge_kernel<TA_><<<n_tokens, TALK_THREADS, 0, stream>>>(ws, (TA_*)out, out_stride,       \
+                                                                                    out_scale, tokens, Hq, Dv, splits); \
     } while (0)
+#define QE_TALK(TA_) do { if (nv == 8) QE_TALK2(TA_, 8); else QE_TALK2(TA_, 16); } while (0)
     if (dt_a == QE_F32) QE_TALK(float);
     else if (dt_a == QE_BF16) QE_TALK(bf16_t);
     else QE_REQUIRE(false, "talking attention: unknown element type %d", dt_a);
 #undef QE_TALK
+#undef QE_TALK2
     QE_LAUNCH_CHECK();
     return 0;
 }

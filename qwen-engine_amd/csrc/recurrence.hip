@@ -285,3 +285,266 @@ extern "C" int qe_scaled_sum(const void* a, float sa, const void* b, float sb, i
     QE_LAUNCH_CHECK();
     return 0;
 }
+
+// ---- the recurrences over long portions, chunk by chunk ---------------------------------------------------
+// A portion of a request's rows is cut into chunks of C rows.  With S the state before a chunk, t and s rows of the
+// chunk, g_s what the chunk's remaining decays make of row s's k v^T at the chunk's end, and a_t what the decays
+// before row t make of S:
+//   S_out = diag(gamma) S + sum_s diag(g_s) k_s v_s^T            o_t = (q_t * a_t)^T S + sum_s A[t][s] v_s
+//   one decay per head:       g_s = decay^(n-1-s), gamma = decay^n, a_t = decay^(t+1), A[t][s] = decay^(t-s) q_t . k_s (s <= t)
+//   a decay per key channel:  with L_t the running sum of log w (= -exp(x + w0)) up to row t, in 64-bit:
+//       g_s = exp(L_(n-1) - L_s), gamma = exp(L_(n-1)), a_t = exp(L_(t-1)),
+//       A[t][s] = sum_d q_t[d] k_s[d] exp(L_(t-1)[d] - L_s[d]) (s < t),  A[t][t] = sum_d q_t[d] u[d] k_t[d]
+//   (every exponent is <= 0: nothing overflows however strong the decays; log w is kept above -200, below which
+//   w is 0 in 32-bit anyway, so that the running sums keep their small terms)
+// Three launches: every chunk's sum_s diag(g_s) k_s v_s^T and gamma (parallel over chunks, heads and blocks of 64
+// value columns); the states before every chunk, chunk after chunk within a portion (elementwise), which also leaves
+// the portion's last state in the request's slot; every chunk's outputs (parallel again).
+// chunks: int32 [n][2] = (first row, rows <= C); portions: int32 [m][3] = (first chunk, chunks, first row); a portion's
+// state row is tok_seq of its first row, read on the device (a recorded step serves another request at every replay).
+#define RC_THREADS 256
+
+struct RecChunkLayout { int ld, d4, q, k, v, a, s, pw, l, total; };   // offsets in floats
+
+__host__ __device__ __forceinline__ RecChunkLayout rec_chunk_layout(int C, int D, int mode) {
+    RecChunkLayout L;
+    L.d4 = (D + 3) & ~3;
+    L.ld = L.d4 + (((L.d4 >> 2) & 1) ? 0 : 4);
+    L.q = 0;
+    L.k = L.q + C * L.ld;
+    L.v = L.k + C * L.ld;
+    L.a = L.v + C * 64;
+    L.s = L.a + C * C;
+    L.pw = L.s + L.d4 * 64;
+    L.l = L.pw + ((C + 1 + 3) & ~3);
+    L.total = L.l + (mode == 1 ? 2 * C * L.d4 : 0);
+    return L;
+}
+
+extern "C" int qe_recurrence_chunk_len(int D) { return D <= 64 ? 64 : (D <= 128 ? 32 : 16); }
+
+// PHASE 0: a chunk's contribution to the state and its whole decay; PHASE 1: its outputs from the state before it
+template <typename TA, int MODE, int PHASE>
+__global__ __launch_bounds__(RC_THREADS) void recurrence_chunk_kernel(
+    const TA* __restrict__ q, const TA* __restrict__ k, const TA* __restrict__ v, long row_stride,
+    const float* __restrict__ wx, long w_stride, const float* __restrict__ w0, const float* __restrict__ u,
+    const float* __restrict__ decay, int act_silu, const int* __restrict__ chunks, float* __restrict__ ws_s,
+    float* __restrict__ ws_g, float* __restrict__ out, int C, int H, int D, int Dv) {
+    extern __shared__ __align__(16) float sm[];
+    const RecChunkLayout L = rec_chunk_layout(C, D, MODE);
+    float* qs = sm + L.q;
+    float* ks = sm + L.k;
+    float* vs = sm + L.v;
+    float* A = sm + L.a;
+    float* Ss = sm + L.s;
+    float* pw = sm + L.pw;
+    double* Ld = (double*)(sm + L.l);
+    const int c = blockIdx.x, h = blockIdx.y, z = blockIdx.z, tid = threadIdx.x;
+    const int row0 = chunks[2 * c], n = chunks[2 * c + 1];
+    const int col0 = z * 64;
+
+    for (int i = tid; i < C * L.d4; i += RC_THREADS) {
+        const int t = i / L.d4, d = i - t * L.d4;
+        float a = 0.f, b = 0.f;
+        double lw = 0.0;
+        if (t < n && d < D) {
+            const long r = (long)(row0 + t) * row_stride + h * D + d;
+            b = Elem<TA>::load(k + r);
+            if (PHASE == 1) a = Elem<TA>::load(q + r);
+            if (act_silu) { a = silu_f(a); b = silu_f(b); }
+            if (MODE == 1) lw = -(double)fminf(expf(wx[(long)(row0 + t) * w_stride + h * D + d] + w0[h * D + d]), 200.f);   // (exp(-200) is 0 in 32-bit)
+        }
+        qs[t * L.ld + d] = a;
+        ks[t * L.ld + d] = b;
+        if (MODE == 1) Ld[t * L.d4 + d] = lw;
+    }
+    for (int i = tid; i < C * 64; i += RC_THREADS) {
+        const int t = i >> 6, cc = i & 63;
+        float x = 0.f;
+        if (t < n && col0 + cc < Dv) {
+            x = Elem<TA>::load(v + (long)(row0 + t) * row_stride + (long)h * Dv + col0 + cc);
+            if (act_silu) x = silu_f(x);
+        }
+        vs[i] = x;
+    }
+    if (MODE == 0 && tid == 0) {
+        float x = 1.f;
+        const float dec = decay[h];
+        for (int i = 0; i <= C; ++i) { pw[i] = x; x *= dec; }
+    }
+    __syncthreads();
+    if (MODE == 1) {
+        for (int d = tid; d < L.d4; d += RC_THREADS) {
+            double run = 0.0;
+            for (int t = 0; t < C; ++t) { run += Ld[t * L.d4 + d]; Ld[t * L.d4 + d] = run; }     // (rows from n on add nothing)
+        }
+        __syncthreads();
+    }
+    const int vq = tid & 15, rq = tid >> 4;                                  // a thread's four columns and row group
+
+    if (PHASE == 0) {
+        for (int i = tid; i < C * L.d4; i += RC_THREADS) {
+            const int s = i / L.d4, d = i - s * L.d4;
+            float g = 0.f;
+            if (s < n) g = MODE == 0 ? pw[n - 1 - s] : expf((float)(Ld[(n - 1) * L.d4 + d] - Ld[s * L.d4 + d]));
+            ks[s * L.ld + d] *= g;
+        }
+        if (z == 0)
+            for (int d = tid; d < D; d += RC_THREADS)
+                ws_g[((long)c * H + h) * D + d] = MODE == 0 ? pw[n] : expf((float)Ld[(n - 1) * L.d4 + d]);
+        __syncthreads();
+        float* dst = ws_s + ((long)c * H + h) * D * Dv;
+        for (int d0 = rq * 4; d0 < L.d4; d0 += 64) {
+            float acc[4][4] = {};
+            for (int s = 0; s < n; ++s) {
+                const float4 kk = *(const float4*)(ks + s * L.ld + d0);
+                const float4 vv = *(const float4*)(vs + s * 64 + vq * 4);
+                const float ka[4] = {kk.x, kk.y, kk.z, kk.w}, va[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(ka[i], va[j], acc[i][j]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int d = d0 + i, cc = col0 + vq * 4 + j;
+                    if (d < D && cc < Dv) dst[(long)d * Dv + cc] = acc[i][j];
+                }
+        }
+        return;
+    }
+
+    // ---- PHASE 1
+    const float* src = ws_s + ((long)c * H + h) * D * Dv;                    // (the state before this chunk by now)
+    for (int i = tid; i < L.d4 * 64; i += RC_THREADS) {
+        const int d = i >> 6, cc = i & 63;
+        Ss[i] = (d < D && col0 + cc < Dv) ? src[(long)d * Dv + col0 + cc] : 0.f;
+    }
+    for (int i = tid; i < C * C; i += RC_THREADS) {
+        const int t = i / C, s = i - t * C;
+        float a = 0.f;
+        if (t < n && s <= t) {
+            const float4* qt = (const float4*)(qs + t * L.ld);
+            const float4* kk = (const float4*)(ks + s * L.ld);
+            if (MODE == 0) {
+                float x = 0.f, y = 0.f;
+                for (int d = 0; d < (L.d4 >> 2); ++d) {
+                    const float4 e = qt[d], f = kk[d];
+                    x = fmaf(e.x, f.x, x); y = fmaf(e.y, f.y, y); x = fmaf(e.z, f.z, x); y = fmaf(e.w, f.w, y);
+                }
+                a = (x + y) * pw[t - s];
+            } else if (s == t) {
+                for (int d = 0; d < D; ++d) a = fmaf(qs[t * L.ld + d] * u[h * D + d], ks[s * L.ld + d], a);
+            } else {
+                const double* lt = Ld + (t - 1) * L.d4;
+                const double* ls = Ld + s * L.d4;
+                for (int d = 0; d < D; ++d)
+                    a = fmaf(qs[t * L.ld + d] * ks[s * L.ld + d], expf((float)(lt[d] - ls[d])), a);
+            }
+        }
+        A[i] = a;
+    }
+    __syncthreads();
+    for (int i = tid; i < C * L.d4; i += RC_THREADS) {
+        const int t = i / L.d4, d = i - t * L.d4;
+        float a;
+        if (MODE == 0) a = pw[t + 1];
+        else a = t == 0 ? 1.f : expf((float)Ld[(t - 1) * L.d4 + d]);
+        qs[t * L.ld + d] *= a;
+    }
+    __syncthreads();
+    for (int t0 = rq * 4; t0 < C; t0 += 64) {
+        if (t0 >= n) break;
+        float acc[4][4] = {};
+        for (int d = 0; d < L.d4; ++d) {
+            const float4 sv = *(const float4*)(Ss + d * 64 + vq * 4);
+            const float sa[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float x = qs[(t0 + i) * L.ld + d];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(x, sa[j], acc[i][j]);
+            }
+        }
+        const int s_end = t0 + 4 < n ? t0 + 4 : n;
+        for (int s = 0; s < s_end; ++s) {
+            const float4 vv = *(const float4*)(vs + s * 64 + vq * 4);
+            const float va[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float x = A[(t0 + i) * C + s];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(x, va[j], acc[i][j]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int t = t0 + i, cc = col0 + vq * 4 + j;
+                if (t < n && cc < Dv) out[((long)(row0 + t) * H + h) * Dv + cc] = acc[i][j];
+            }
+    }
+}
+
+// grid (portions, H, blocks of 256 state numbers): S_in of every chunk replaces the chunk's contribution in ws_s
+__global__ void recurrence_scan_kernel(const int* __restrict__ portions, const int* __restrict__ tok_seq,
+                                       float* __restrict__ ws_s,
+                                       const float* __restrict__ ws_g, float* __restrict__ state, long state_stride,
+                                       int H, int D, int Dv) {
+    const int e = blockIdx.z * blockDim.x + threadIdx.x;
+    if (e >= D * Dv) return;
+    const int pi = blockIdx.x, h = blockIdx.y, d = e / Dv;
+    const int c0 = portions[3 * pi], nc = portions[3 * pi + 1], slot = tok_seq[portions[3 * pi + 2]];
+    float* sp = state + (long)slot * state_stride + (long)h * D * Dv + e;
+    float S = *sp;
+    for (int c = c0; c < c0 + nc; ++c) {
+        float* w = ws_s + ((long)c * H + h) * D * Dv + e;
+        const float add = *w;
+        *w = S;
+        S = fmaf(ws_g[((long)c * H + h) * D + d], S, add);
+    }
+    *sp = S;
+}
+
+// As qe_linear_recurrence, for rows cut into chunks of C = qe_recurrence_chunk_len(D) rows on the host.  ws: float32,
+// n_chunks * H * (D * Dv + D) numbers.  Rows that no chunk names are left alone.
+extern "C" int qe_linear_recurrence_chunked(const void* q, const void* k, const void* v, long row_stride, const float* wx,
+                                            long w_stride, const float* w0, const float* u, const float* decay, int mode,
+                                            int act_silu, float* state, long state_stride, const int* tok_seq,
+                                            const int* chunks, int n_chunks, const int* portions, int n_portions, float* ws, float* out,
+                                            int H, int D, int Dv, int dt_a, hipStream_t stream) {
+    QE_REQUIRE(n_chunks >= 0 && n_portions >= 0 && H > 0 && D > 0 && Dv > 0, "linear_recurrence: bad sizes");
+    QE_REQUIRE(D <= 256, "linear_recurrence: heads of %d key channels (at most 256)", D);
+    QE_REQUIRE(mode == 0 ? decay != nullptr : (mode == 1 && wx && w0 && u), "linear_recurrence: mode %d lacks operands", mode);
+    QE_REQUIRE(state_stride >= (long)H * D * Dv, "linear_recurrence: state rows overlap");
+    if (n_chunks == 0) return 0;
+    QE_REQUIRE(ws && chunks && portions, "linear_recurrence: chunks without a workspace");
+    const int C = qe_recurrence_chunk_len(D);
+    const RecChunkLayout L = rec_chunk_layout(C, D, mode);
+    const size_t shmem = (size_t)L.total * sizeof(float);
+    QE_REQUIRE(shmem <= 150 * 1024, "linear_recurrence: %zu bytes of shared memory", shmem);
+    float* ws_s = ws;
+    float* ws_g = ws + (long)n_chunks * H * D * Dv;
+    dim3 grid(n_chunks, H, (Dv + 63) / 64);
+#define QE_RC(TA_, MODE_, PHASE_)                                                                                    \
+    do {                                                                                                             \
+        if (shmem > 48 * 1024)                                                                                       \
+            (void)hipFuncSetAttribute((const void*)recurrence_chunk_kernel<TA_, MODE_, PHASE_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
+        recurrence_chunk_kernel<TA_, MODE_, PHASE_><<<grid, RC_THREADS, shmem, stream>>>(                            \
+            (const TA_*)q, (const TA_*)k, (const TA_*)v, row_stride, wx, w_stride, w0, u, decay, act_silu, chunks,   \
+            ws_s, ws_g, out, C, H, D, Dv);                                                                           \
+    } while (0)
+#define QE_RC2(TA_, PHASE_) do { if (mode == 0) QE_RC(TA_, 0, PHASE_); else QE_RC(TA_, 1, PHASE_); } while (0)
+    QE_REQUIRE(dt_a == QE_F32 || dt_a == QE_BF16, "linear_recurrence: unknown element type %d", dt_a);
+    if (dt_a == QE_F32) QE_RC2(float, 0); else QE_RC2(bf16_t, 0);
+    recurrence_scan_kernel<<<dim3(n_portions, H, (D * Dv + 255) / 256), 256, 0, stream>>>(portions, tok_seq, ws_s, ws_g, state,
+                                                                                         state_stride, H, D, Dv);
+    if (dt_a == QE_F32) QE_RC2(float, 1); else QE_RC2(bf16_t, 1);
+#undef QE_RC2
+#undef QE_RC
+    QE_LAUNCH_CHECK();
+    return 0;
+}

@@ -89,8 +89,12 @@ def load_library():
         "qe_qkv_norm_store": [vp, i32, vp, vp, i32, f32, i32, i32, f32, vp, vp, i32, vp, vp, i32, vp, vp, vp,
                               i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_attention_talk": [vp, vp, i64, f32, vp, vp, vp, vp, i32, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32,
-                              f32, i32, i32, vp],
+                              f32, i32, i32, vp, i32, vp],
+        "qe_attention_talk_splits": [i32, i32],
         "qe_token_shift": [vp, vp, i32, vp, i64, vp, vp, i32, i32, i32, i32, vp],
+        "qe_recurrence_chunk_len": [i32],
+        "qe_linear_recurrence_chunked": [vp, vp, vp, i64, vp, i64, vp, vp, vp, i32, i32, vp, i64, vp, vp, i32, vp, i32, vp, vp,
+                                         i32, i32, i32, i32, vp],
         "qe_linear_recurrence": [vp, vp, vp, i64, vp, i64, vp, vp, vp, i32, i32, vp, i64, vp, vp, i32, i32, i32, i32,
                                  i32, vp],
         "qe_gated_norm": [vp, vp, vp, i64, i32, i32, f32, f32, vp, i64, i32, i32, i32, i32, vp],
@@ -1363,10 +1367,16 @@ def attention_talk(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor
     if tokens is not None:
         _need(tokens, "tokens", torch.int32, (None,), dev)
         n_tok = tokens.shape[0]
+    # a token's keys are dealt to several blocks while the tokens alone do not fill the machine
+    splits = lib.qe_attention_talk_splits(n_tok, -int(window) if window < 0 else int(window))
+    ws = None
+    if splits > 1:
+        ws = torch.empty((n_tok * splits * (2 * Hq + n),), dtype=torch.float32, device=dev)
     _check(lib.qe_attention_talk(q.data_ptr(), out.data_ptr(), out.stride(0) if T > 1 else n, float(out_scale),
                                  cache.data_ptr(), positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
                                  block_table.shape[1], _ptr(tokens), n_tok, _ptr(bias), rows, _ptr(talk), Hq, Hkv,
-                                 int(k_dim), int(v_dim), Dc, P, float(scale), int(window), _DT[q.dtype], _stream()),
+                                 int(k_dim), int(v_dim), Dc, P, float(scale), int(window), int(splits), _ptr(ws),
+                                 _DT[q.dtype], _stream()),
            "attention_talk")
     return out
 
@@ -1398,16 +1408,35 @@ def _rows_view(t: torch.Tensor, name: str, n: int, T: int):
     return t.stride(0) if T > 1 else n
 
 
+def recurrence_chunk_len(head_dim: int) -> int:
+    """Rows of a chunk of the chunked recurrence for heads of this many key channels."""
+    return load_library().qe_recurrence_chunk_len(int(head_dim))
+
+
+def recurrence_chunks(portions, chunk_len: int):
+    """For portions given as (first row, rows) on the host: the ``chunks`` of linear_recurrence(), a pair of int32
+    tensors (on the host) [n, 2] = (first row, rows <= chunk_len) and [m, 3] = (first chunk, chunks, first row)."""
+    chunks, ports = [], []
+    for start, n in portions:
+        if n <= 0:
+            continue
+        ports.append((len(chunks), -(-n // chunk_len), start))
+        chunks += [(start + r, min(chunk_len, n - r)) for r in range(0, n, chunk_len)]
+    return (torch.tensor(chunks, dtype=torch.int32).view(-1, 2), torch.tensor(ports, dtype=torch.int32).view(-1, 3))
+
+
 def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, tok_seq: torch.Tensor,
                       heads: int, decay: Optional[torch.Tensor] = None, decay_x: Optional[torch.Tensor] = None,
                       decay_bias: Optional[torch.Tensor] = None, bonus: Optional[torch.Tensor] = None,
-                      silu: bool = False) -> torch.Tensor:
+                      silu: bool = False, chunks=None) -> torch.Tensor:
     """Per head, with a 32-bit state S [D][Dv] per request (state[tok_seq[t]], float32 [slots, >= H D Dv]):
     with ``decay`` (float32 [H]):  S <- decay_h S + k_t v_t^T, o_t = S^T q_t;
     with ``decay_x`` float32 [T, H D], ``decay_bias`` and ``bonus`` (float32 [H D]):  o_t = (S + diag(bonus) k_t v_t^T)^T q_t,
     then S <- diag(w_t) S + k_t v_t^T with w_t = exp(-exp(decay_x_t + decay_bias)).
     q, k [T, H D], v [T, H Dv] (column slices of one wider tensor are taken as they are, all with one row stride);
-    ``silu``: the three pass silu first.  Returns o float32 [T, H, Dv]."""
+    ``silu``: the three pass silu first.  Returns o float32 [T, H, Dv].
+    ``chunks`` (recurrence_chunks() of all rows' portions, on the device, for recurrence_chunk_len(D)): the rows are
+    taken chunk by chunk, the chunks in parallel, instead of row by row: for long portions."""
     lib = load_library()
     T, dev, H = q.shape[0], q.device, int(heads)
     if q.dtype not in _ACT or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -1430,6 +1459,17 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: 
         _need(decay_bias, "decay_bias", torch.float32, (H * D,), dev)
         _need(bonus, "bonus", torch.float32, (H * D,), dev)
     out = torch.empty((T, H, Dv), dtype=torch.float32, device=dev)
+    if chunks is not None and chunks[0].shape[0]:
+        ch, po = chunks
+        _need(ch, "chunks", torch.int32, (None, 2), dev)
+        _need(po, "portions", torch.int32, (None, 3), dev)
+        ws = torch.empty((ch.shape[0] * H * (D * Dv + D),), dtype=torch.float32, device=dev)
+        _check(lib.qe_linear_recurrence_chunked(q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, _ptr(decay_x), sw,
+                                                _ptr(decay_bias), _ptr(bonus), _ptr(decay), mode, int(bool(silu)),
+                                                state.data_ptr(), state.stride(0), tok_seq.data_ptr(), ch.data_ptr(),
+                                                ch.shape[0], po.data_ptr(), po.shape[0], ws.data_ptr(), out.data_ptr(),
+                                                H, D, Dv, _DT[q.dtype], _stream()), "linear_recurrence (chunked)")
+        return out
     _check(lib.qe_linear_recurrence(q.data_ptr(), k.data_ptr(), v.data_ptr(), sq, _ptr(decay_x), sw, _ptr(decay_bias),
                                     _ptr(bonus), _ptr(decay), mode, int(bool(silu)), state.data_ptr(), state.stride(0),
                                     tok_seq.data_ptr(), out.data_ptr(), T, H, D, Dv, _DT[q.dtype], _stream()),

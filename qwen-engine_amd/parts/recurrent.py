@@ -18,6 +18,24 @@ def _single_rows(ctx, T: int) -> bool:
     return len(ctx.seqs) == T and all(s.q_len == 1 for s in ctx.seqs)
 
 
+# From this many rows of one request in a step, the recurrences take the step's rows chunk by chunk (the chunks in
+# parallel) instead of row by row.
+CHUNKED_FROM_ROWS = 64
+
+
+def _chunks(ctx, head_dim: int):
+    """The step's rows cut into chunks for the chunked recurrence, if a request brings many rows: built and sent to the
+    device once per step and chunk length, shared by the layers.  None: row by row."""
+    if max((s.q_len for s in ctx.seqs), default=0) < CHUNKED_FROM_ROWS:
+        return None
+    C = ops.recurrence_chunk_len(head_dim)
+    key = ("recurrence.chunks", C)
+    if key not in ctx.memo:
+        ch, po = ops.recurrence_chunks([(s.q_start, s.q_len) for s in ctx.seqs], C)
+        ctx.memo[key] = (ch.to(ctx.rt.device), po.to(ctx.rt.device))
+    return ctx.memo[key]
+
+
 class ShiftedDecayMixer:
     """``ShiftedDecaySpec``: five blends of each token with the token before it, projections r, k, v, a silu gate
     and a decay per key channel through a low rank, the recurrence with a bonus for the token itself, a norm per
@@ -72,7 +90,7 @@ class ShiftedDecayMixer:
         low = ops.unary(ops.gemm(m[4], self.w_1, out_dtype=torch.float32), ops.UNARY_TANH, out_dtype=ctx.rt.dtype)
         decay_x = ops.gemm(low, self.w_2, out_dtype=torch.float32)      # (exponentials of the decay: in the recurrence, 32-bit)
         o = ops.linear_recurrence(r, k, v, st[:, W:], ctx.tok_seq, self.h, decay_x=decay_x, decay_bias=self.w0,
-                                  bonus=self.u)
+                                  bonus=self.u, chunks=_chunks(ctx, self.d))
         y = ops.gated_norm(o.view(T, self.h * self.d), self.norm, self.eps, self.h, ctx.rt.dtype, gate=gate,
                            gate_act=ops.GATE_SILU)
         return ops.gemm(y, self.w_o, out_dtype=torch.float32)
@@ -122,7 +140,7 @@ class DecayedLinearMixer:
         nk, nv = self.h * self.d, self.h * self.dv
         y = ops.gemm(x, self.w_in)
         o = ops.linear_recurrence(y[:, :nk], y[:, nk:2 * nk], y[:, 2 * nk:2 * nk + nv], binding.state, ctx.tok_seq,
-                                  self.h, decay=self.decay, silu=True)
+                                  self.h, decay=self.decay, silu=True, chunks=_chunks(ctx, self.d))
         z = ops.gated_norm(o.view(T, nv), self.norm, self.eps, 1, ctx.rt.dtype, gate=y[:, 2 * nk + nv:],
                            gate_act=ops.GATE_SIGMOID)
         return ops.gemm(z, self.w_o, out_dtype=torch.float32)

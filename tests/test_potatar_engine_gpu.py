@@ -95,7 +95,7 @@ def test_bfloat16_agrees_with_the_plain_model_and_with_itself_in_every_cutting(f
         traces.run_in_process(trace, folders[which], "bfloat16", out, page)
         got[cut] = traces.collect(trace, out, cfg["vocab"])
         # (with alpha 1 a mixer's rounding weighs as much as the stream: twice the allowance against 64-bit)
-        _assert_bfloat16_close(got[cut], ref, f"{cut} against the plain model", median=4e-2, largest=2e-1)
+        _assert_bfloat16_close(got[cut], ref, f"{cut} against the plain model", median=4e-2, largest=5e-1)
     whole = {rid: torch.stack([torch.from_numpy(got["whole"][rid][p]) for p in range(len(t))]) for rid, t in reqs.items()}
     for cut in ("mixed", "portions", "tail"):
         _assert_bfloat16_close(got[cut], whole, f"{cut} against whole prompts")

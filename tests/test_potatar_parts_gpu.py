@@ -312,6 +312,15 @@ REC_STEPS = [[(0, 5), (1, 1), (2, 2)], [(1, 1), (0, 1)], [(2, 1)], [(2, 37), (0,
 REC_LENGTHS = {0: 176, 1: 7, 2: 111}
 
 
+def _chunks_of(portions, head_dim, chunked):
+    """The chunk lists of a step's portions for the chunked path (the kernels then take the rows chunk by chunk, the
+    chunks in parallel), or None for the path that walks row by row."""
+    if not chunked:
+        return None
+    ch, po = ops().recurrence_chunks(portions, ops().recurrence_chunk_len(head_dim))
+    return ch.to(DEV), po.to(DEV)
+
+
 def _run_recurrence(call, inputs, widths, slot, out_cols):
     """Feeds the requests' rows through ``call`` in REC_STEPS; returns each request's outputs in order."""
     done = {s: 0 for s in REC_LENGTHS}
@@ -323,7 +332,11 @@ def _run_recurrence(call, inputs, widths, slot, out_cols):
             for i, t in enumerate(inputs):
                 rows[i].append(t[s][done[s]:done[s] + n])
             seq += [slot[s]] * n
-        out = call([torch.cat(r).to(DEV) for r in rows], i32(seq))
+        starts, at = [], 0
+        for _, n in step:
+            starts.append((at, n))
+            at += n
+        out = call([torch.cat(r).to(DEV) for r in rows], i32(seq), starts)
         at = 0
         for s, n in step:
             got[s].append(out[at:at + n].cpu())
@@ -337,7 +350,8 @@ def _run_recurrence(call, inputs, widths, slot, out_cols):
 @pytest.mark.parametrize("H,D,Dv,decay", [(2, 12, 8, (0.5, 0.93)), (4, 32, 64, (0.6, 0.88, 0.97, 0.999)), (2, 64, 128, (0.8, 0.99)),
                                           (3, 4, 20, (1.0, 0.5, 0.25)), (1, 16, 16, (1.0,)), (2, 128, 128, (0.0, 0.9)),
                                           (1, 24, 200, (0.95,))])
-def test_recurrence_with_a_decay_per_head_across_cuts_and_slots(dtype, tol, H, D, Dv, decay):
+@pytest.mark.parametrize("chunked", [False, True])
+def test_recurrence_with_a_decay_per_head_across_cuts_and_slots(dtype, tol, H, D, Dv, decay, chunked):
     """(the inputs are rounded to the activation type first, the recurrence itself is 32-bit in both: one tolerance)"""
     o = ops()
     g = torch.Generator().manual_seed(H * D)
@@ -349,10 +363,10 @@ def test_recurrence_with_a_decay_per_head_across_cuts_and_slots(dtype, tol, H, D
         state[s, :nk * Dv] = 0
     dec = torch.tensor(decay, dtype=torch.float64)
 
-    def call(rows, seq):
+    def call(rows, seq, portions):
         r = rows[0]
         return o.linear_recurrence(r[:, :nk], r[:, nk:2 * nk], r[:, 2 * nk:2 * nk + nv], state, seq, H,
-                                   decay=dec.float().to(DEV), silu=True)
+                                   decay=dec.float().to(DEV), silu=True, chunks=_chunks_of(portions, D, chunked))
 
     got = _run_recurrence(call, [y], None, slot, nv)
     for s, n in REC_LENGTHS.items():
@@ -365,7 +379,8 @@ def test_recurrence_with_a_decay_per_head_across_cuts_and_slots(dtype, tol, H, D
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-5)])
 @pytest.mark.parametrize("H,D", [(3, 8), (2, 32), (2, 64), (1, 16), (5, 64), (1, 128), (2, 20)])
-def test_recurrence_with_a_decay_per_channel_and_a_bonus_across_cuts_and_slots(dtype, tol, H, D):
+@pytest.mark.parametrize("chunked", [False, True])
+def test_recurrence_with_a_decay_per_channel_and_a_bonus_across_cuts_and_slots(dtype, tol, H, D, chunked):
     o = ops()
     g = torch.Generator().manual_seed(H * D + 1)
     slot = {0: 1, 1: 3, 2: 0}
@@ -374,6 +389,7 @@ def test_recurrence_with_a_decay_per_channel_and_a_bonus_across_cuts_and_slots(d
     k = {s: torch.randn(n, n_, generator=g).to(dtype) for s, n in REC_LENGTHS.items()}
     v = {s: torch.randn(n, n_, generator=g).to(dtype) for s, n in REC_LENGTHS.items()}
     wx = {s: torch.randn(n, n_, generator=g) * 1.5 for s, n in REC_LENGTHS.items()}      # decays from nearly 0 to nearly 1
+    wx[0][40:44] = 95.0                                           # (and decays of exactly 0: exp(95) is beyond 32-bit)
     w0 = torch.randn(n_, generator=g) * 0.8 - 1.0
     u = torch.randn(n_, generator=g) * 0.5
     W = 9                                                         # (the state's first numbers belong to the blends)
@@ -381,9 +397,9 @@ def test_recurrence_with_a_decay_per_channel_and_a_bonus_across_cuts_and_slots(d
     for s in slot.values():
         state[s, W:] = 0
 
-    def call(rows, seq):
+    def call(rows, seq, portions):
         return o.linear_recurrence(rows[0], rows[1], rows[2], state[:, W:], seq, H, decay_x=rows[3], decay_bias=w0.to(DEV),
-                                   bonus=u.to(DEV))
+                                   bonus=u.to(DEV), chunks=_chunks_of(portions, D, chunked))
 
     got = _run_recurrence(call, [r, k, v, wx], None, slot, n_)
     for s, n in REC_LENGTHS.items():
@@ -394,7 +410,8 @@ def test_recurrence_with_a_decay_per_channel_and_a_bonus_across_cuts_and_slots(d
     assert torch.isnan(state[2]).all() and torch.isnan(state[:, :W]).all()
 
 
-def test_a_state_far_back_is_kept_or_forgotten():
+@pytest.mark.parametrize("chunked", [False, True])
+def test_a_state_far_back_is_kept_or_forgotten(chunked):
     """One early token writes a large k v^T; hundreds of tokens later a query along that key reads it back: whole with a
     decay of 1, scaled by decay^n otherwise.  Random inputs alone would bury a lost state under the recent tokens."""
     o = ops()
@@ -412,7 +429,7 @@ def test_a_state_far_back_is_kept_or_forgotten():
         outs, at = [], 0
         for m in cut:
             outs.append(o.linear_recurrence(q[at:at + m].to(DEV), k[at:at + m].to(DEV), v[at:at + m].to(DEV), state, i32([0] * m), H,
-                                            decay=dec.to(DEV)))
+                                            decay=dec.to(DEV), chunks=_chunks_of([(0, m)], D, chunked)))
             at += m
         assert rel(torch.cat(outs), want) < 2e-5, cut
 
