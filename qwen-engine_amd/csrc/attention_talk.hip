@@ -4,12 +4,16 @@
 //   o_h(i)    = sum_j softmax_j(s'_h(i, .)) v(j)
 // Both the bias and the mixing are optional.  Because a head's weights depend on every head's scores against a
 // key, one block handles all heads of one token.  Keys are walked 64 at a time from the first key the token sees
-// (first_seen_key: all, a window of the last keys, or the token's own chunk).  For a tile of 64 keys the block
-//   - brings the key rows of as many key/value heads as fit a staging buffer into shared memory (contiguous loads,
-//     converted to 32-bit, rows padded so that a lane per key reads its row without bank conflicts), and every
-//     wave takes query heads in turn, a lane per key, for the dot products;
-//   - mixes the heads' scores and takes the tile into each head's running softmax (a wave per head);
-//   - brings the value rows into the same buffer and adds the tile's values, a thread per output number.
+// (first_seen_key: all, a window of the last keys, or the token's own chunk).  A tile of 64 keys goes through a
+// staging buffer in shared memory in stages, each brought in by contiguous loads and converted to 32-bit, the loads
+// of the next stage (or of the next tile's first) in flight while the block computes on the present one:
+//   - the key rows of as many key/value heads as fit (rows padded so that a lane per key reads its row without bank
+//     conflicts): every wave takes query heads in turn, a lane per key, for the dot products; the biases of a
+//     tile are loaded a tile ahead;
+//   - after the last stage of keys the heads' scores are mixed and the tile joins each head's running softmax (a
+//     wave per head);
+//   - the value rows of all key/value heads for as many of the tile's keys as fit: a thread per four neighbouring
+//     output numbers adds the stage's values.
 // With KS > 1 the tiles of a token are dealt to KS blocks in turn; each leaves its maxima, sums and accumulators in a
 // workspace and attention_talk_merge_kernel weighs and adds them in the order of the splits.  The order of the sums
 // depends on the position and KS alone: not on how the request was cut into steps.  All arithmetic in 32-bit.
@@ -44,12 +48,12 @@ struct TalkLayout {              // offsets into shared memory, in floats (all m
     int rs_q, ls_k, ls_v, stage, sc, pm, small, total;
 };
 
-__host__ __device__ __forceinline__ TalkLayout talk_layout(int Hq, int Dk, int Dv, int HGk, int HGv) {
+__host__ __device__ __forceinline__ TalkLayout talk_layout(int Hq, int Hkv, int Dk, int Dv, int HGk, int KPS) {
     TalkLayout L;
     L.rs_q = (Dk + 3) & ~3;
     L.ls_k = L.rs_q + (((L.rs_q >> 2) & 1) ? 0 : 4);      // an odd number of 16-byte pieces a row
     L.ls_v = (Dv + 3) & ~3;
-    const int a = HGk * 64 * L.ls_k, b = HGv * 64 * L.ls_v;
+    const int a = HGk * 64 * L.ls_k, b = Hkv * KPS * L.ls_v;
     L.stage = 256 + Hq * L.rs_q;                           // (256 floats = twice 64 offsets of 8 bytes come first)
     L.sc = L.stage + (a > b ? a : b);
     L.pm = L.sc + Hq * 64;
@@ -58,31 +62,33 @@ __host__ __device__ __forceinline__ TalkLayout talk_layout(int Hq, int Dk, int D
     return L;
 }
 
-// A stage: the rows of `hg` key/value heads from g0, of one plane, of a tile's 64 keys.  talk_fetch starts the
-// loads of a stage into registers (NV pieces of four numbers a thread; keys that are not seen, offset < 0, become
-// zeros); talk_commit writes them to stage[gl][jj][ls] in 32-bit.  Between the two the block computes on the stage
-// before.
-// item[u]: (row of the stage << 8) | piece of the row, for the thread's u-th piece of a stage; -1: beyond a full stage
+// A stage of keys: the key rows of `hg` key/value heads from g0 for the tile's 64 keys (row gl * 64 + jj).  A stage of
+// values: the value rows of all key/value heads for KPS of the tile's keys from k0 (row gl * KPS + jl), so that every
+// thread has work in every stage.  talk_fetch starts the loads of a stage into registers (NV pieces of four numbers a
+// thread; keys that are not seen, offset < 0, become zeros); talk_commit writes them to the staging buffer in 32-bit.
+// Between the two the block computes on the stage before.
+// item[u]: (row of the stage << 8) | piece of the row, for the thread's u-th piece of a full stage; -1: beyond it
 template <int NV>
-__device__ __forceinline__ void talk_items(int (&item)[NV], int hmax, int vec_per_row) {
+__device__ __forceinline__ void talk_items(int (&item)[NV], int rows, int vec_per_row) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
         const int i = threadIdx.x + u * TALK_THREADS;
-        item[u] = i < hmax * 64 * vec_per_row ? ((i / vec_per_row) << 8) | (i % vec_per_row) : -1;
+        item[u] = i < rows * vec_per_row ? ((i / vec_per_row) << 8) | (i % vec_per_row) : -1;
     }
 }
 
+// rows: of this stage (<= those of a full one); a row's key is k0 + (row & (2^kshift - 1)), its head g0 + (row >> kshift)
 template <typename TA, int NV>
 __device__ __forceinline__ void talk_fetch(typename Raw4<TA>::R (&regs)[NV], const int (&item)[NV],
-                                           const TA* __restrict__ plane, const long* koff, int g0, int hg,
-                                           long head_stride) {
+                                           const TA* __restrict__ plane, const long* koff, int g0, int rows, int kshift,
+                                           int k0, long head_stride) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
         typename Raw4<TA>::R r = Raw4<TA>::zero();
         const int rr = item[u] >> 8;
-        if (item[u] >= 0 && rr < hg * 64) {
-            const long off = koff[rr & 63];
-            if (off >= 0) r = Raw4<TA>::load(plane + off + (long)(g0 + (rr >> 6)) * head_stride + (item[u] & 255) * 4);
+        if (item[u] >= 0 && rr < rows) {
+            const long off = koff[k0 + (rr & ((1 << kshift) - 1))];
+            if (off >= 0) r = Raw4<TA>::load(plane + off + (long)(g0 + (rr >> kshift)) * head_stride + (item[u] & 255) * 4);
         }
         regs[u] = r;
     }
@@ -90,14 +96,16 @@ __device__ __forceinline__ void talk_fetch(typename Raw4<TA>::R (&regs)[NV], con
 
 template <typename TA, int NV>
 __device__ __forceinline__ void talk_commit(const typename Raw4<TA>::R (&regs)[NV], const int (&item)[NV],
-                                            float* stage, int hg, int ls) {
+                                            float* stage, int rows, int ls) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
         const int rr = item[u] >> 8;
-        if (item[u] >= 0 && rr < hg * 64)
-            *(float4*)(stage + (long)rr * ls + (item[u] & 255) * 4) = Raw4<TA>::widen(regs[u]);      // (rr = gl * 64 + jj)
+        if (item[u] >= 0 && rr < rows)
+            *(float4*)(stage + (long)rr * ls + (item[u] & 255) * 4) = Raw4<TA>::widen(regs[u]);
     }
 }
+
+#define TALK_BIAS_PRE 8          // a thread's first heads' biases for the next tile are loaded a tile ahead
 
 template <typename TA, int NV>
 __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
@@ -105,9 +113,10 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
     const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ tokens, const float* __restrict__ bias, int bias_rows,
     const float* __restrict__ talk, int Hq, int Hkv, int Dk, int Dv, int Dc, int P, float scale, int window,
-    int KS, int HGk, int HGv, float* __restrict__ ws) {
+    int KS, int HGk, int kps_shift, float* __restrict__ ws) {
     extern __shared__ __align__(16) float sm[];
-    const TalkLayout L = talk_layout(Hq, Dk, Dv, HGk, HGv);
+    const int KPS = 1 << kps_shift;
+    const TalkLayout L = talk_layout(Hq, Hkv, Dk, Dv, HGk, KPS);
     long* koff = (long*)sm;                       // twice 64 key rows: this tile's and the next one's (-1: not seen)
     float* qs = sm + 256;                         // Hq rows of rs_q
     float* stage = sm + L.stage;
@@ -125,7 +134,7 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
     const int* bt = block_table + (long)tok_seq[t] * max_blocks;
     const long page_stride = 2L * Hkv * P * Dc, plane = (long)Hkv * P * Dc, head_stride = (long)P * Dc;
     const int n_out = Hq * Dv;
-    const int nK = (Hkv + HGk - 1) / HGk, nS = nK + (Hkv + HGv - 1) / HGv;      // stages of a tile: keys, then values
+    const int nK = (Hkv + HGk - 1) / HGk, nS = nK + (64 >> kps_shift);           // stages of a tile: keys, then values
     const int vpr_k = L.rs_q >> 2, vpr_v = L.ls_v >> 2;
 
     for (int i = tid; i < Hq * L.rs_q; i += TALK_THREADS) {
@@ -145,17 +154,21 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
     }
     typename Raw4<TA>::R regs[NV];
     int item_k[NV], item_v[NV];
-    talk_items<NV>(item_k, HGk, vpr_k);
-    talk_items<NV>(item_v, HGv, vpr_v);
+    talk_items<NV>(item_k, HGk * 64, vpr_k);
+    talk_items<NV>(item_v, Hkv * KPS, vpr_v);
+    float bpre[TALK_BIAS_PRE];                     // biases of heads wave, wave + 4, ... against this lane's key
 
     int j0 = lo + 64 * split, par = 0;
     if (j0 <= p) {
-        if (wave == 0) {
-            const int j = j0 + lane;
-            koff[lane] = j <= p ? (long)bt[j / P] * page_stride + (long)(j % P) * Dc : -1L;
+        const int j = j0 + lane;
+        if (wave == 0) koff[lane] = j <= p ? (long)bt[j / P] * page_stride + (long)(j % P) * Dc : -1L;
+#pragma unroll
+        for (int i = 0; i < TALK_BIAS_PRE; ++i) {
+            const int h = wave + 4 * i, n = p - j;
+            bpre[i] = (bias && j <= p && h < Hq) ? bias[(long)(n < bias_rows ? n : bias_rows - 1) * Hq + h] : 0.f;
         }
         __syncthreads();
-        talk_fetch<TA, NV>(regs, item_k, cache, koff, 0, Hkv < HGk ? Hkv : HGk, head_stride);
+        talk_fetch<TA, NV>(regs, item_k, cache, koff, 0, (Hkv < HGk ? Hkv : HGk) * 64, 6, 0, head_stride);
     }
     for (; j0 <= p; j0 += 64 * KS, par ^= 1) {
         const long* ko = koff + par * 64;
@@ -165,29 +178,56 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
         const int j = j0 + lane;
         const bool seen = j <= p;
         if (wave == 0) kn[lane] = jn + lane <= p ? (long)bt[(jn + lane) / P] * page_stride + (long)((jn + lane) % P) * Dc : -1L;
+        float bnow[TALK_BIAS_PRE];
+#pragma unroll
+        for (int i = 0; i < TALK_BIAS_PRE; ++i) bnow[i] = bpre[i];
         for (int s = 0; s < nS; ++s) {
             const bool is_v = s >= nK;
-            const int g0 = is_v ? (s - nK) * HGv : s * HGk;
-            const int hmax = is_v ? HGv : HGk;
-            const int hg = Hkv - g0 < hmax ? Hkv - g0 : hmax;
+            const int g0 = is_v ? 0 : s * HGk;
+            const int hg = is_v ? Hkv : (Hkv - g0 < HGk ? Hkv - g0 : HGk);
+            const int k0 = is_v ? (s - nK) << kps_shift : 0;
             __syncthreads();                                 // (the stage before has been read)
-            if (is_v) talk_commit<TA, NV>(regs, item_v, stage, hg, L.ls_v);
-            else talk_commit<TA, NV>(regs, item_k, stage, hg, L.ls_k);
+            if (is_v) talk_commit<TA, NV>(regs, item_v, stage, Hkv * KPS, L.ls_v);
+            else talk_commit<TA, NV>(regs, item_k, stage, hg * 64, L.ls_k);
             if (s + 1 < nS) {                                // the next stage's loads fly while this one is computed on
-                const bool nv = s + 1 >= nK;
-                const int n0 = nv ? (s + 1 - nK) * HGv : (s + 1) * HGk;
-                const int nmax = nv ? HGv : HGk;
-                const int nh = Hkv - n0 < nmax ? Hkv - n0 : nmax;
-                if (nv) talk_fetch<TA, NV>(regs, item_v, cache + plane, ko, n0, nh, head_stride);
-                else talk_fetch<TA, NV>(regs, item_k, cache, ko, n0, nh, head_stride);
+                if (s + 1 >= nK) {
+                    talk_fetch<TA, NV>(regs, item_v, cache + plane, ko, 0, Hkv * KPS, kps_shift, (s + 1 - nK) << kps_shift,
+                                       head_stride);
+                } else {
+                    const int n0 = (s + 1) * HGk;
+                    talk_fetch<TA, NV>(regs, item_k, cache, ko, n0, (Hkv - n0 < HGk ? Hkv - n0 : HGk) * 64, 6, 0, head_stride);
+                }
             } else if (more) {
-                talk_fetch<TA, NV>(regs, item_k, cache, kn, 0, Hkv < HGk ? Hkv : HGk, head_stride);
+                talk_fetch<TA, NV>(regs, item_k, cache, kn, 0, (Hkv < HGk ? Hkv : HGk) * 64, 6, 0, head_stride);
+#pragma unroll
+                for (int i = 0; i < TALK_BIAS_PRE; ++i) {
+                    const int h = wave + 4 * i, n = p - (jn + lane);
+                    bpre[i] = (bias && n >= 0 && h < Hq) ? bias[(long)(n < bias_rows ? n : bias_rows - 1) * Hq + h] : 0.f;
+                }
             }
             __syncthreads();
             if (!is_v) {
                 // ---- scores: thread (wave, lane) takes heads wave, wave + 4, ... of the staged key heads against key j
-                for (int h = g0 * G + wave; h < (g0 + hg) * G; h += TALK_THREADS / 64) {
-                    const float4* kr = (const float4*)(stage + (long)((h / G - g0) * 64 + lane) * L.ls_k);
+#pragma unroll
+                for (int i = 0; i < TALK_BIAS_PRE; ++i) {
+                    const int h = wave + 4 * i, gk = h / G;
+                    if (h < Hq && gk >= g0 && gk < g0 + hg) {
+                        const float4* kr = (const float4*)(stage + (long)((gk - g0) * 64 + lane) * L.ls_k);
+                        const float4* qh = (const float4*)(qs + h * L.rs_q);
+                        float d0 = 0.f, d1 = 0.f;
+#pragma unroll 4
+                        for (int d = 0; d < vpr_k; ++d) {
+                            const float4 a = qh[d], b = kr[d];
+                            d0 = fmaf(a.x, b.x, d0); d1 = fmaf(a.y, b.y, d1);
+                            d0 = fmaf(a.z, b.z, d0); d1 = fmaf(a.w, b.w, d1);
+                        }
+                        sc[h * 64 + lane] = (d0 + d1) * scale + bnow[i];
+                    }
+                }
+                for (int h = wave + 4 * TALK_BIAS_PRE; h < Hq; h += TALK_THREADS / 64) {      // (more than 32 heads)
+                    const int gk = h / G;
+                    if (gk < g0 || gk >= g0 + hg) continue;
+                    const float4* kr = (const float4*)(stage + (long)((gk - g0) * 64 + lane) * L.ls_k);
                     const float4* qh = (const float4*)(qs + h * L.rs_q);
                     float d0 = 0.f, d1 = 0.f;
                     for (int d = 0; d < vpr_k; ++d) {
@@ -224,17 +264,17 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
                     }
                 }
             } else {
-                // ---- the tile's values (unseen keys: zeros with weight zero)
+                // ---- the stage's values (unseen keys: zeros with weight zero)
 #pragma unroll
                 for (int i = 0; i < TALK_MAX_ACC; ++i) {
-                    const int h = hd[i] >> 16, gk = h / G;
-                    if (h < Hq && gk >= g0 && gk < g0 + hg) {
-                        const float* vs = stage + (long)(gk - g0) * 64 * L.ls_v + (hd[i] & 0xffff);
-                        const float4* ph = (const float4*)(pm + h * 64);
-                        const float f = al[h];
+                    const int h = hd[i] >> 16;
+                    if (h < Hq) {
+                        const float* vs = stage + (long)(h / G) * KPS * L.ls_v + (hd[i] & 0xffff);
+                        const float4* ph = (const float4*)(pm + h * 64 + k0);
+                        const float f = k0 == 0 ? al[h] : 1.f;
                         float4 a = make_float4(acc[i].x * f, acc[i].y * f, acc[i].z * f, acc[i].w * f);
-#pragma unroll 4
-                        for (int jj = 0; jj < 16; ++jj) {
+#pragma unroll 2
+                        for (int jj = 0; jj < (KPS >> 2); ++jj) {
                             const float4 w = ph[jj];
                             const float wa[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
@@ -329,14 +369,17 @@ extern "C" int qe_attention_talk(const void* q, void* out, long out_stride, floa
     QE_REQUIRE(out_stride >= (long)Hq * Dv, "talking attention: output rows overlap");
     QE_REQUIRE(splits >= 1 && splits <= TALK_MAX_SPLITS && (splits == 1 || ws), "talking attention: %d splits", splits);
     if (n_tokens == 0) return 0;
-    const TalkLayout L0 = talk_layout(Hq, Dk, Dv, 1, 1);
+    const TalkLayout L0 = talk_layout(Hq, Hkv, Dk, Dv, 1, 4);
     const int vk = L0.rs_q >> 2, vv = L0.ls_v >> 2;
-    QE_REQUIRE(vk <= 64 && vv <= 64, "talking attention: heads of %d and %d numbers (at most 256)", Dk, Dv);
-    const int nv = (vk > 32 || vv > 32) ? 16 : 8;           // pieces a thread holds of a stage: 256 * nv pieces a stage
-    int hgk = 4 * nv / vk, hgv = 4 * nv / vv;
+    QE_REQUIRE(vk <= 64, "talking attention: key heads of %d numbers (at most 256)", Dk);
+    QE_REQUIRE((long)Hkv * 4 * vv <= TALK_THREADS * 16, "talking attention: %d value heads of %d numbers", Hkv, Dv);
+    // pieces a thread holds of a stage (256 * nv pieces a stage)
+    const int nv = (vk > 32 || (long)Hkv * 4 * vv > TALK_THREADS * 8) ? 16 : 8;
+    int hgk = 4 * nv / vk;
     hgk = hgk > Hkv ? Hkv : hgk;
-    hgv = hgv > Hkv ? Hkv : hgv;
-    const TalkLayout L = talk_layout(Hq, Dk, Dv, hgk, hgv);
+    int kps_shift = 6;                                      // keys of a stage of values: a power of two from 4 to 64
+    while (kps_shift > 2 && ((long)Hkv << kps_shift) * vv > TALK_THREADS * nv) --kps_shift;
+    const TalkLayout L = talk_layout(Hq, Hkv, Dk, Dv, hgk, 1 << kps_shift);
     const size_t shmem = (size_t)L.total * sizeof(float);
     QE_REQUIRE(shmem <= 150 * 1024, "talking attention: %zu bytes of shared memory", shmem);
     dim3 grid(n_tokens, splits);
@@ -346,7 +389,7 @@ extern "C" int qe_attention_talk(const void* q, void* out, long out_stride, floa
             (void)hipFuncSetAttribute((const void*)attention_talk_kernel<TA_, NV_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
         attention_talk_kernel<TA_, NV_><<<grid, TALK_THREADS, shmem, stream>>>(                                      \
             (const TA_*)q, (TA_*)out, out_stride, out_scale, (const TA_*)cache, positions, tok_seq, block_table,     \
-            max_blocks, tokens, bias, bias_rows, talk, Hq, Hkv, Dk, Dv, Dc, P, scale, window, splits, hgk, hgv, ws); \
+            max_blocks, tokens, bias, bias_rows, talk, Hq, Hkv, Dk, Dv, Dc, P, scale, window, splits, hgk, kps_shift, ws); \
         if (splits > 1)                                                                                              \
             attention_talk_merge_kernel<TA_><<<n_tokens, TALK_THREADS, 0, stream>>>(ws, (TA_*)out, out_stride,       \
                                                                                     out_scale, tokens, Hq, Dv, splits); \
