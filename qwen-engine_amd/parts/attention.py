@@ -408,24 +408,32 @@ class ConvAttention(PagedAttention):
         return self._project_out(o)
 
 
-def distance_bias_rows(table: torch.Tensor, far: float) -> torch.Tensor:
+def distance_bias_rows(table: torch.Tensor, far: float, max_distance: Optional[int] = None) -> torch.Tensor:
     """A learned bias by distance as one row per distance: ``table`` [B, heads] holds a row each for the distances
     below B // 2 and logarithmic steps up to ``far`` for the rest; distance n reads row n for n < B // 2, else
     min(B - 1, B // 2 + floor(log(n / (B // 2)) / log(far / (B // 2)) * (B - B // 2))).  Returns float32
     [ceil(far) + 1, heads]: row n for distance n, the last row for every distance beyond (it is the table's last).
-    The rows are looked up in 64-bit on the host, once."""
+    With ``max_distance`` (the largest distance a query ever has to a key it sees, a chunk's length less one) the
+    rows end there.  The rows are looked up in 64-bit on the host, once."""
     import math
     B = table.shape[0]
     half = B // 2
     if half < 1 or not far > half:
         raise ValueError(f"a distance bias of {B} rows up to {far}")
     rows = []
-    for n in range(int(math.ceil(far)) + 1):
+    count = int(math.ceil(far)) + 1
+    if max_distance is not None and max_distance + 1 < count:
+        count = int(max_distance) + 1
+        far_row = None
+    else:
+        far_row = B - 1
+    for n in range(count):
         if n < half:
             rows.append(n)
         else:
             rows.append(min(B - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (B - half)))))
-    rows[-1] = B - 1
+    if far_row is not None:
+        rows[-1] = far_row
     return table.float()[torch.tensor(rows)].contiguous()
 
 
@@ -524,7 +532,8 @@ class ChunkAttention(PagedAttention):
         if s.value_blend == "blend":
             self.blend = rt.place_vector(tensors[s.blend_name].reshape(1))
         if s.distance_bias_rows:
-            self.dist_bias = rt.place_vector(distance_bias_rows(tensors[s.distance_bias_name], float(s.distance_bias_far)))
+            self.dist_bias = rt.place_vector(distance_bias_rows(tensors[s.distance_bias_name], float(s.distance_bias_far),
+                                                                max_distance=self.chunk - 1 if self.chunk else None))
         if s.talking_heads:
             self.talk = rt.place_vector(tensors[s.talk_name])
         w_o = tensors[no]

@@ -136,6 +136,9 @@ def test_bias_rows_by_distance(rows, far):
     assert torch.equal(got[-1], table[-1])
     for n in (got.shape[0], 3 * got.shape[0], 100000):           # (beyond the last row: the table's last)
         assert N.distance_bucket(n, rows, far) == rows - 1
+    short = distance_bias_rows(table, far, max_distance=3)        # (a chunk of four positions: distances 0 to 3)
+    assert torch.equal(short, got[:4]) if got.shape[0] > 4 else torch.equal(short, got)
+    assert torch.equal(distance_bias_rows(table, 1e9, max_distance=50)[50], table[N.distance_bucket(50, rows, 1e9)])
 
 
 # ---- attention whose heads talk, inside chunks, over pages ---------------------------------------------------------
