@@ -197,7 +197,8 @@ extern "C" int qe_linear_recurrence(const void* q, const void* k, const void* v,
 }
 
 // ---- norm, gate --------------------------------------------------------------------------------------
-// One block per row, a wave per group in turn.  gate_act: 0 none, 1 silu, 2 sigmoid.
+// One block per row, a wave per group in turn; fewer groups than waves: all waves share every group's sums through
+// shared memory.  gate_act: 0 none, 1 silu, 2 sigmoid.
 template <typename TG, typename TO>
 __global__ void gated_norm_kernel(const float* __restrict__ o, const float* __restrict__ weight,
                                   const TG* __restrict__ gate, long gate_stride, int gate_act, float eps, float scale,
@@ -205,6 +206,31 @@ __global__ void gated_norm_kernel(const float* __restrict__ o, const float* __re
     const long t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int n = N / groups;
+    if (groups < nw) {
+        __shared__ float part[16];
+        for (int g = 0; g < groups; ++g) {
+            const float* og = o + t * N + (long)g * n;
+            float a = 0.f;
+            for (int c = threadIdx.x; c < n; c += blockDim.x) a += og[c] * og[c];
+            a = wave_sum(a);
+            __syncthreads();                                 // (the group before has been read)
+            if (lane == 0) part[wave] = a;
+            __syncthreads();
+            float all = 0.f;
+            for (int w = 0; w < nw; ++w) all += part[w];     // (every thread adds in the order of the waves)
+            const float f = rsqrtf(all / (float)n + eps);
+            for (int c = threadIdx.x; c < n; c += blockDim.x) {
+                const int cc = g * n + c;
+                float val = og[c] * f * weight[cc];
+                if (gate) {
+                    const float z = Elem<TG>::load(gate + t * gate_stride + cc);
+                    val *= gate_act == 1 ? silu_f(z) : (gate_act == 2 ? sigmoid_f(z) : z);
+                }
+                Elem<TO>::store(y + t * y_stride + cc, val * scale);
+            }
+        }
+        return;
+    }
     for (int g = wave; g < groups; g += nw) {
         const float* og = o + t * N + (long)g * n;
         float a = 0.f;
@@ -229,7 +255,7 @@ extern "C" int qe_gated_norm(const float* o, const float* weight, const void* ga
     QE_REQUIRE(T >= 0 && N > 0 && groups > 0 && N % groups == 0, "gated_norm: rows of %d in %d groups", N, groups);
     QE_REQUIRE(y_stride >= N && (!gate || gate_stride >= N), "gated_norm: rows overlap");
     if (T == 0) return 0;
-    const int threads = groups >= 4 ? 256 : 64 * groups;
+    const int threads = (groups >= 4 || N / groups >= 512) ? 256 : 64 * groups;   // (long groups: four waves share each)
 #define QE_GN(TG_, TO_) gated_norm_kernel<TG_, TO_><<<T, threads, 0, stream>>>(o, weight, (const TG_*)gate, gate_stride, gate_act, eps, scale, (TO_*)y, y_stride, N, groups)
     const int dg = gate ? dt_g : dt_y;
     if (dg == QE_F32 && dt_y == QE_F32) QE_GN(float, float);

@@ -438,7 +438,7 @@ def test_a_state_far_back_is_kept_or_forgotten(chunked):
 
 
 # ---- norm and gate after a recurrence -----------------------------------------------------------------------------------
-@pytest.mark.parametrize("T,N_,groups", [(5, 24, 3), (9, 256, 1), (3, 640, 5), (2, 2048, 16), (1, 20, 1)])
+@pytest.mark.parametrize("T,N_,groups", [(5, 24, 3), (9, 256, 1), (3, 640, 5), (2, 2048, 16), (1, 20, 1), (4, 1024, 1), (2, 1200, 2)])
 @pytest.mark.parametrize("act", ["silu", "sigmoid", None])
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-6), (torch.bfloat16, 6e-3)])
 def test_norm_and_gate(T, N_, groups, act, dtype, tol):
