@@ -25,6 +25,7 @@
 #define TALK_THREADS 256
 #define TALK_MAX_ACC 4           // groups of four outputs a thread: Hq * ceil(Dv / 4) <= 256 * 4
 #define TALK_MAX_SPLITS 16
+#define TALK_ROWS 4              // rows a block of the kernel for many rows
 
 // Four consecutive elements as they lie in memory, and as four floats.
 template <typename T> struct Raw4;
@@ -317,6 +318,261 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_kernel(
     }
 }
 
+// ---- several rows a block ------------------------------------------------------------------------------------
+// For portions of prompts: a block takes R neighbouring rows of the flat batch.  Rows of one request whose first seen
+// key is the same (one chunk, or no window) are walked together over the keys up to the last row's position, so that
+// a stage of keys or values is brought in once for all of them, a key's numbers are read once for R dot products, and a
+// value's once for R sums; every row masks the keys behind its own position.  Rows of the block that belong
+// elsewhere (another request, the next chunk) get a pass of their own.  Everything else as in the kernel above.
+struct TalkRowsLayout { int stage, sc, pm, small, total; };
+
+__host__ __device__ __forceinline__ TalkRowsLayout talk_rows_layout(const TalkLayout& L1, int R, int Hq) {
+    TalkRowsLayout L;
+    const int stage_floats = L1.sc - L1.stage;
+    L.stage = 256 + R * Hq * L1.rs_q;
+    L.sc = L.stage + stage_floats;
+    L.pm = L.sc + R * Hq * 64;
+    L.small = L.pm + R * Hq * 64;
+    L.total = L.small + ((3 * R * Hq + Hq * Hq + 3) & ~3);
+    return L;
+}
+
+template <typename TA, int NV, int R>
+__global__ __launch_bounds__(TALK_THREADS) void attention_talk_rows_kernel(
+    const TA* __restrict__ q, TA* __restrict__ out, long out_stride, float out_scale, const TA* __restrict__ cache,
+    const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
+    int max_blocks, int T, const float* __restrict__ bias, int bias_rows, const float* __restrict__ talk, int Hq,
+    int Hkv, int Dk, int Dv, int Dc, int P, float scale, int window, int KS, int HGk, int kps_shift,
+    float* __restrict__ ws) {
+    extern __shared__ __align__(16) float sm[];
+    const int KPS = 1 << kps_shift;
+    const TalkLayout L = talk_layout(Hq, Hkv, Dk, Dv, HGk, KPS);
+    const TalkRowsLayout LR = talk_rows_layout(L, R, Hq);
+    long* koff = (long*)sm;
+    float* qs = sm + 256;                         // R * Hq rows of rs_q
+    float* stage = sm + LR.stage;
+    float* sc = sm + LR.sc;                       // R * Hq * 64 scores
+    float* pm = sm + LR.pm;                       // R * Hq * 64 weights
+    float* ml = sm + LR.small;                    // R * Hq * 2 running maximum and sum
+    float* al = ml + 2 * R * Hq;                  // R * Hq factors of the tile
+    float* tk = al + R * Hq;                      // Hq * Hq (if talk)
+    const int split = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int G = Hq / Hkv;
+    const long page_stride = 2L * Hkv * P * Dc, plane = (long)Hkv * P * Dc, head_stride = (long)P * Dc;
+    const int n_out = Hq * Dv;
+    const int nK = (Hkv + HGk - 1) / HGk, nS = nK + (64 >> kps_shift);
+    const int vpr_k = L.rs_q >> 2, vpr_v = L.ls_v >> 2;
+    const long row0 = (long)blockIdx.x * R;
+
+    int pr[R], sq[R], lo_r[R];                     // (the same in every thread)
+    unsigned todo = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        pr[r] = 0; sq[r] = -1; lo_r[r] = 0;
+        if (row0 + r < T) {
+            pr[r] = positions[row0 + r];
+            sq[r] = tok_seq[row0 + r];
+            lo_r[r] = first_seen_key(pr[r], window);
+            todo |= 1u << r;
+        }
+    }
+    if (talk) for (int i = tid; i < Hq * Hq; i += TALK_THREADS) tk[i] = talk[i];
+    int hd[TALK_MAX_ACC];
+#pragma unroll
+    for (int i = 0; i < TALK_MAX_ACC; ++i) {
+        const int o = tid + i * TALK_THREADS;
+        const int h = o < Hq * vpr_v ? o / vpr_v : Hq;
+        hd[i] = (h << 16) | (h < Hq ? (o - h * vpr_v) * 4 : 0);
+    }
+    int item_k[NV], item_v[NV];
+    talk_items<NV>(item_k, HGk * 64, vpr_k);
+    talk_items<NV>(item_v, Hkv * KPS, vpr_v);
+    typename Raw4<TA>::R regs[NV];
+
+    while (todo) {
+        // ---- the rows of this pass: the first row left and every later one of its request with its first seen key
+        const int lead = __ffs(todo) - 1;
+        unsigned grp = 0;
+        int p_max = 0;
+        const int lo = lo_r[lead];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if ((todo >> r & 1u) && sq[r] == sq[lead] && lo_r[r] == lo) {
+                grp |= 1u << r;
+                p_max = pr[r] > p_max ? pr[r] : p_max;
+            }
+        todo &= ~grp;
+        const int* bt = block_table + (long)sq[lead] * max_blocks;
+        __syncthreads();                                     // (the pass before has left shared memory)
+        for (int i = tid; i < R * Hq * L.rs_q; i += TALK_THREADS) {
+            const int rh = i / L.rs_q, d = i - rh * L.rs_q, r = rh / Hq, h = rh - r * Hq;
+            qs[i] = ((grp >> r & 1u) && d < Dk) ? Elem<TA>::load(q + ((row0 + r) * Hq + h) * Dc + d) : 0.f;
+        }
+        for (int i = tid; i < R * Hq; i += TALK_THREADS) { ml[2 * i] = -INFINITY; ml[2 * i + 1] = 0.f; }
+        float4 acc[TALK_MAX_ACC][R];
+#pragma unroll
+        for (int i = 0; i < TALK_MAX_ACC; ++i)
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[i][r] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+        int j0 = lo + 64 * split, par = 0;
+        if (j0 <= p_max) {
+            const int j = j0 + lane;
+            if (wave == 0) koff[lane] = j <= p_max ? (long)bt[j / P] * page_stride + (long)(j % P) * Dc : -1L;
+            __syncthreads();
+            talk_fetch<TA, NV>(regs, item_k, cache, koff, 0, (Hkv < HGk ? Hkv : HGk) * 64, 6, 0, head_stride);
+        }
+        for (; j0 <= p_max; j0 += 64 * KS, par ^= 1) {
+            const long* ko = koff + par * 64;
+            long* kn = koff + (par ^ 1) * 64;
+            const int jn = j0 + 64 * KS;
+            const bool more = jn <= p_max;
+            const int j = j0 + lane;
+            if (wave == 0) kn[lane] = jn + lane <= p_max ? (long)bt[(jn + lane) / P] * page_stride + (long)((jn + lane) % P) * Dc : -1L;
+            for (int s = 0; s < nS; ++s) {
+                const bool is_v = s >= nK;
+                const int g0 = is_v ? 0 : s * HGk;
+                const int hg = is_v ? Hkv : (Hkv - g0 < HGk ? Hkv - g0 : HGk);
+                const int k0 = is_v ? (s - nK) << kps_shift : 0;
+                __syncthreads();
+                if (is_v) talk_commit<TA, NV>(regs, item_v, stage, Hkv * KPS, L.ls_v);
+                else talk_commit<TA, NV>(regs, item_k, stage, hg * 64, L.ls_k);
+                if (s + 1 < nS) {
+                    if (s + 1 >= nK) {
+                        talk_fetch<TA, NV>(regs, item_v, cache + plane, ko, 0, Hkv * KPS, kps_shift, (s + 1 - nK) << kps_shift,
+                                           head_stride);
+                    } else {
+                        const int n0 = (s + 1) * HGk;
+                        talk_fetch<TA, NV>(regs, item_k, cache, ko, n0, (Hkv - n0 < HGk ? Hkv - n0 : HGk) * 64, 6, 0, head_stride);
+                    }
+                } else if (more) {
+                    talk_fetch<TA, NV>(regs, item_k, cache, kn, 0, (Hkv < HGk ? Hkv : HGk) * 64, 6, 0, head_stride);
+                }
+                __syncthreads();
+                if (!is_v) {
+                    // ---- scores of R rows: a key's numbers are read once for the R dot products
+                    for (int h = g0 * G + wave; h < (g0 + hg) * G; h += TALK_THREADS / 64) {
+                        float bv[R];
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+                            const int n = pr[r] - j;
+                            bv[r] = (bias && (grp >> r & 1u) && n >= 0) ? bias[(long)(n < bias_rows ? n : bias_rows - 1) * Hq + h] : 0.f;
+                        }
+                        const float4* kr = (const float4*)(stage + (long)((h / G - g0) * 64 + lane) * L.ls_k);
+                        float dt[R];
+#pragma unroll
+                        for (int r = 0; r < R; ++r) dt[r] = 0.f;
+#pragma unroll 2
+                        for (int d = 0; d < vpr_k; ++d) {
+                            const float4 b = kr[d];
+#pragma unroll
+                            for (int r = 0; r < R; ++r) {
+                                const float4 a = *(const float4*)(qs + (r * Hq + h) * L.rs_q + d * 4);
+                                dt[r] = fmaf(a.x, b.x, dt[r]); dt[r] = fmaf(a.y, b.y, dt[r]);
+                                dt[r] = fmaf(a.z, b.z, dt[r]); dt[r] = fmaf(a.w, b.w, dt[r]);
+                            }
+                        }
+#pragma unroll
+                        for (int r = 0; r < R; ++r) sc[(r * Hq + h) * 64 + lane] = dt[r] * scale + bv[r];
+                    }
+                    if (s == nK - 1) {
+                        __syncthreads();
+                        // ---- the heads' scores mixed, then the tile joins each row's and head's running softmax
+                        for (int rh = wave; rh < R * Hq; rh += TALK_THREADS / 64) {
+                            const int r = rh / Hq, h = rh - r * Hq;
+                            if (!(grp >> r & 1u) || j0 > pr[r]) {            // not a row of this pass, or none of its keys here
+                                pm[rh * 64 + lane] = 0.f;
+                                if (lane == 0) al[rh] = 1.f;
+                                continue;
+                            }
+                            const bool seen = j <= pr[r];
+                            float sv;
+                            if (talk) {
+                                sv = 0.f;
+                                for (int g = 0; g < Hq; ++g) sv = fmaf(tk[h * Hq + g], sc[(r * Hq + g) * 64 + lane], sv);
+                            } else {
+                                sv = sc[rh * 64 + lane];
+                            }
+                            if (!seen) sv = -INFINITY;
+                            const float m_old = ml[2 * rh], l_old = ml[2 * rh + 1];
+                            const float m_new = fmaxf(m_old, wave_max(sv));  // finite: key j0 is seen by this row
+                            const float a = expf(m_old - m_new);
+                            const float pj = seen ? expf(sv - m_new) : 0.f;
+                            const float l_new = l_old * a + wave_sum(pj);
+                            pm[rh * 64 + lane] = pj;
+                            if (lane == 0) { ml[2 * rh] = m_new; ml[2 * rh + 1] = l_new; al[rh] = a; }
+                        }
+                    }
+                } else {
+                    // ---- the stage's values: a value's numbers are read once for the R sums
+#pragma unroll
+                    for (int i = 0; i < TALK_MAX_ACC; ++i) {
+                        const int h = hd[i] >> 16;
+                        if (h < Hq) {
+                            const float* vs = stage + (long)(h / G) * KPS * L.ls_v + (hd[i] & 0xffff);
+                            float4 a[R];
+#pragma unroll
+                            for (int r = 0; r < R; ++r) {
+                                const float f = k0 == 0 ? al[r * Hq + h] : 1.f;
+                                a[r] = make_float4(acc[i][r].x * f, acc[i][r].y * f, acc[i][r].z * f, acc[i][r].w * f);
+                            }
+                            for (int jj = 0; jj < KPS; jj += 4) {
+                                float4 w[R];
+#pragma unroll
+                                for (int r = 0; r < R; ++r) w[r] = *(const float4*)(pm + (r * Hq + h) * 64 + k0 + jj);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    const float4 vv = *(const float4*)(vs + (long)(jj + e) * L.ls_v);
+#pragma unroll
+                                    for (int r = 0; r < R; ++r) {
+                                        const float we = e == 0 ? w[r].x : (e == 1 ? w[r].y : (e == 2 ? w[r].z : w[r].w));
+                                        a[r].x = fmaf(we, vv.x, a[r].x); a[r].y = fmaf(we, vv.y, a[r].y);
+                                        a[r].z = fmaf(we, vv.z, a[r].z); a[r].w = fmaf(we, vv.w, a[r].w);
+                                    }
+                                }
+                            }
+#pragma unroll
+                            for (int r = 0; r < R; ++r) acc[i][r] = a[r];
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // ---- the pass's rows leave their results
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!(grp >> r & 1u)) continue;
+            const long t = row0 + r;
+            if (KS == 1) {
+#pragma unroll
+                for (int i = 0; i < TALK_MAX_ACC; ++i) {
+                    const int h = hd[i] >> 16, d = hd[i] & 0xffff;
+                    if (h < Hq) {
+                        const float f = out_scale / ml[2 * (r * Hq + h) + 1];
+                        const float a[4] = {acc[i][r].x, acc[i][r].y, acc[i][r].z, acc[i][r].w};
+                        for (int e = 0; e < 4; ++e)
+                            if (d + e < Dv) Elem<TA>::store(out + t * out_stride + h * Dv + d + e, a[e] * f);
+                    }
+                }
+            } else {
+                float* w = ws + (t * KS + split) * (2 * Hq + n_out);
+                for (int i = tid; i < 2 * Hq; i += TALK_THREADS) w[i] = ml[2 * r * Hq + i];
+#pragma unroll
+                for (int i = 0; i < TALK_MAX_ACC; ++i) {
+                    const int h = hd[i] >> 16, d = hd[i] & 0xffff;
+                    if (h < Hq) {
+                        const float a[4] = {acc[i][r].x, acc[i][r].y, acc[i][r].z, acc[i][r].w};
+                        for (int e = 0; e < 4; ++e)
+                            if (d + e < Dv) w[2 * Hq + h * Dv + d + e] = a[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
 // grid (tokens): the splits' partial results weighed by exp(m_s - max m) and added in the order of the splits
 template <typename TA>
 __global__ __launch_bounds__(TALK_THREADS) void attention_talk_merge_kernel(
@@ -383,6 +639,23 @@ extern "C" int qe_attention_talk(const void* q, void* out, long out_stride, floa
     const size_t shmem = (size_t)L.total * sizeof(float);
     QE_REQUIRE(shmem <= 150 * 1024, "talking attention: %zu bytes of shared memory", shmem);
     dim3 grid(n_tokens, splits);
+    // many rows (portions of prompts): several neighbouring rows a block, where shared memory holds their scores
+    const int R = TALK_ROWS;
+    const TalkRowsLayout LR = talk_rows_layout(L, R, Hq);
+    const size_t shmem_rows = (size_t)LR.total * sizeof(float);
+    const bool rows = !tokens && n_tokens >= 64 && nv == 8 && shmem_rows <= 100 * 1024 &&
+                      (long)Hq * vv <= TALK_THREADS * 2;
+#define QE_TALK_ROWS(TA_)                                                                                            \
+    do {                                                                                                             \
+        if (shmem_rows > 48 * 1024)                                                                                  \
+            (void)hipFuncSetAttribute((const void*)attention_talk_rows_kernel<TA_, 8, TALK_ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem_rows); \
+        attention_talk_rows_kernel<TA_, 8, TALK_ROWS><<<dim3((n_tokens + R - 1) / R, splits), TALK_THREADS, shmem_rows, stream>>>( \
+            (const TA_*)q, (TA_*)out, out_stride, out_scale, (const TA_*)cache, positions, tok_seq, block_table,     \
+            max_blocks, n_tokens, bias, bias_rows, talk, Hq, Hkv, Dk, Dv, Dc, P, scale, window, splits, hgk, kps_shift, ws); \
+        if (splits > 1)                                                                                              \
+            attention_talk_merge_kernel<TA_><<<n_tokens, TALK_THREADS, 0, stream>>>(ws, (TA_*)out, out_stride,       \
+                                                                                    out_scale, tokens, Hq, Dv, splits); \
+    } while (0)
 #define QE_TALK2(TA_, NV_)                                                                                           \
     do {                                                                                                             \
         if (shmem > 48 * 1024)                                                                                       \
@@ -394,12 +667,13 @@ extern "C" int qe_attention_talk(const void* q, void* out, long out_stride, floa
             attention_talk_merge_kernel<TA_><<<n_tokens, TALK_THREADS, 0, stream>>>(ws, (TA_*)out, out_stride,       \
                                                                                     out_scale, tokens, Hq, Dv, splits); \
     } while (0)
-#define QE_TALK(TA_) do { if (nv == 8) QE_TALK2(TA_, 8); else QE_TALK2(TA_, 16); } while (0)
+#define QE_TALK(TA_) do { if (rows) QE_TALK_ROWS(TA_); else if (nv == 8) QE_TALK2(TA_, 8); else QE_TALK2(TA_, 16); } while (0)
     if (dt_a == QE_F32) QE_TALK(float);
     else if (dt_a == QE_BF16) QE_TALK(bf16_t);
     else QE_REQUIRE(false, "talking attention: unknown element type %d", dt_a);
 #undef QE_TALK
 #undef QE_TALK2
+#undef QE_TALK_ROWS
     QE_LAUNCH_CHECK();
     return 0;
 }
