@@ -23,7 +23,8 @@
 #include "common.h"
 
 #define TALK_THREADS 256
-#define TALK_MAX_ACC 4           // groups of four outputs a thread: Hq * ceil(Dv / 4) <= 256 * 4
+#define TALK_MAX_ACC 8           // groups of four outputs a thread: Hq * ceil(Dv / 4) <= 256 * 8
+#define TALK_ROWS_ACC 2          // the same in the kernel for many rows, which holds them for every row of the block
 #define TALK_MAX_SPLITS 16
 #define TALK_ROWS 4              // rows a block of the kernel for many rows
 
@@ -378,9 +379,9 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_rows_kernel(
         }
     }
     if (talk) for (int i = tid; i < Hq * Hq; i += TALK_THREADS) tk[i] = talk[i];
-    int hd[TALK_MAX_ACC];
+    int hd[TALK_ROWS_ACC];
 #pragma unroll
-    for (int i = 0; i < TALK_MAX_ACC; ++i) {
+    for (int i = 0; i < TALK_ROWS_ACC; ++i) {
         const int o = tid + i * TALK_THREADS;
         const int h = o < Hq * vpr_v ? o / vpr_v : Hq;
         hd[i] = (h << 16) | (h < Hq ? (o - h * vpr_v) * 4 : 0);
@@ -410,9 +411,9 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_rows_kernel(
             qs[i] = ((grp >> r & 1u) && d < Dk) ? Elem<TA>::load(q + ((row0 + r) * Hq + h) * Dc + d) : 0.f;
         }
         for (int i = tid; i < R * Hq; i += TALK_THREADS) { ml[2 * i] = -INFINITY; ml[2 * i + 1] = 0.f; }
-        float4 acc[TALK_MAX_ACC][R];
+        float4 acc[TALK_ROWS_ACC][R];
 #pragma unroll
-        for (int i = 0; i < TALK_MAX_ACC; ++i)
+        for (int i = 0; i < TALK_ROWS_ACC; ++i)
 #pragma unroll
             for (int r = 0; r < R; ++r) acc[i][r] = make_float4(0.f, 0.f, 0.f, 0.f);
 
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_rows_kernel(
                 } else {
                     // ---- the stage's values: a value's numbers are read once for the R sums
 #pragma unroll
-                    for (int i = 0; i < TALK_MAX_ACC; ++i) {
+                    for (int i = 0; i < TALK_ROWS_ACC; ++i) {
                         const int h = hd[i] >> 16;
                         if (h < Hq) {
                             const float* vs = stage + (long)(h / G) * KPS * L.ls_v + (hd[i] & 0xffff);
@@ -547,7 +548,7 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_rows_kernel(
             const long t = row0 + r;
             if (KS == 1) {
 #pragma unroll
-                for (int i = 0; i < TALK_MAX_ACC; ++i) {
+                for (int i = 0; i < TALK_ROWS_ACC; ++i) {
                     const int h = hd[i] >> 16, d = hd[i] & 0xffff;
                     if (h < Hq) {
                         const float f = out_scale / ml[2 * (r * Hq + h) + 1];
@@ -560,7 +561,7 @@ __global__ __launch_bounds__(TALK_THREADS) void attention_talk_rows_kernel(
                 float* w = ws + (t * KS + split) * (2 * Hq + n_out);
                 for (int i = tid; i < 2 * Hq; i += TALK_THREADS) w[i] = ml[2 * r * Hq + i];
 #pragma unroll
-                for (int i = 0; i < TALK_MAX_ACC; ++i) {
+                for (int i = 0; i < TALK_ROWS_ACC; ++i) {
                     const int h = hd[i] >> 16, d = hd[i] & 0xffff;
                     if (h < Hq) {
                         const float a[4] = {acc[i][r].x, acc[i][r].y, acc[i][r].z, acc[i][r].w};
@@ -644,7 +645,7 @@ extern "C" int qe_attention_talk(const void* q, void* out, long out_stride, floa
     const TalkRowsLayout LR = talk_rows_layout(L, R, Hq);
     const size_t shmem_rows = (size_t)LR.total * sizeof(float);
     const bool rows = !tokens && n_tokens >= 64 && nv == 8 && shmem_rows <= 100 * 1024 &&
-                      (long)Hq * vv <= TALK_THREADS * 2;
+                      (long)Hq * vv <= TALK_THREADS * TALK_ROWS_ACC;
 #define QE_TALK_ROWS(TA_)                                                                                            \
     do {                                                                                                             \
         if (shmem_rows > 48 * 1024)                                                                                  \

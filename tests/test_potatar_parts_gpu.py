@@ -163,7 +163,7 @@ def _paged(k, v, P, pages, g, dtype, dc, start=0):
     (1, 1, 16, 16, 1, 4, 9, True, True), (16, 1, 8, 8, 1000, 4, 413, True, True), (3, 1, 64, 64, 70, 16, 150, False, True),
     (5, 5, 12, 20, 64, 8, 129, True, False), (16, 4, 64, 64, 256, 16, 600, True, True), (2, 1, 128, 128, 33, 16, 100, True, True),
     (40, 5, 8, 8, 30, 8, 70, True, True), (2, 1, 256, 256, 50, 16, 120, True, True), (12, 12, 36, 36, 90, 16, 200, True, True),
-    (8, 8, 128, 128, 100, 16, 150, True, True)])
+    (8, 8, 128, 128, 100, 16, 150, True, True), (24, 4, 32, 200, 50, 16, 90, True, True), (32, 8, 64, 160, 70, 16, 100, True, True)])
 def test_talking_heads_attention_with_a_bias_by_distance(dtype, tol, hq, hkv, dk, dv, chunk, P, n, bias, talk):
     """Every position of a sequence at once (a prompt), then positions alone (decoded tokens) and in a batch beside
     another request whose pages lie between this one's."""
