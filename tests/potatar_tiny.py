@@ -54,7 +54,7 @@ SHAPE_SIZES["A"] = {0: 5, 2: 10}
 PB = {"architecture": "Potatar", "vocab": 300, "width": 128, "norm": {"eps": 1e-5}, "postln_alpha": 3.0, "logit_softcap": 30.0,
       "layers": [
           parallel(4, 4, 64, 40, 0.12, 100.5, 2, 64, 128, (0.8, 0.99), 1.5, 0.5, ff(96)),
-          attention(8, 2, 64, 64, 40, 32, 0.11, True, 500000.0, ff(64)),
+          attention(8, 2, 64, 64, 40, 16, 0.11, True, 200000.0, ff(64)),
           wkv(2, 64, None),
           attention(2, 2, 128, 64, 100, 64, 0.08, True, 10000.0, ff(128)),
       ]}

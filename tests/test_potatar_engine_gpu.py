@@ -321,7 +321,7 @@ def test_command_line_with_random_weights(tmp_path, capsys):
 PM = {"architecture": "Potatar", "vocab": 701, "width": 320, "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "logit_softcap": 20.0,
       "layers": [
           attention(6, 2, 64, 40, 150, 24, 0.12, True, 20000.0, ff(256)),
-          parallel(8, 2, 32, 150, 0.2, 200, 4, 32, 64, (0.7, 0.9, 0.97, 0.999), 1.1, 0.9, ff(128)),
+          parallel(8, 2, 32, 150, 0.2, 200, 4, 24, 48, (0.7, 0.9, 0.96, 0.998), 1.1, 0.9, ff(128)),
           wkv(5, 64, None),
           attention(4, 2, 128, 40, 333, 128, 0.09, True, 3000.0, ff(192)),
           parallel(3, 1, 64, 70, 0.13, 64, 2, 64, 40, (0.95, 0.5), 0.8, 1.2, None),

@@ -27,7 +27,7 @@ def i32(v):
 
 
 # ---- the norm after the sum ------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("T,W,alpha", [(1, 80, 1.7), (9, 192, 2.5), (70, 1024, 1.0), (3, 4100, 0.3)])
+@pytest.mark.parametrize("T,W,alpha", [(1, 80, 1.7), (9, 200, 2.25), (70, 1024, 1.0), (3, 4100, 0.3)])
 @pytest.mark.parametrize("ddtype", [torch.float32, torch.bfloat16])
 def test_norm_after_the_sum(T, W, alpha, ddtype):
     g = torch.Generator().manual_seed(T + W)
@@ -46,7 +46,7 @@ def test_activations_between_products_and_the_soft_cap():
     o = ops()
     assert rel(o.unary(z.to(DEV), o.UNARY_GELU), N.gelu_erf(z.double())) < 2e-6
     assert rel(o.unary(z.to(DEV), o.UNARY_TANH), torch.tanh(z.double())) < 2e-6
-    for cap in (1.0, 15.0, 40.0):
+    for cap in (1.0, 12.0, 40.0):
         assert rel(o.unary((5 * z).to(DEV), o.UNARY_SOFTCAP, cap=cap), cap * torch.tanh(5 * z.double() / cap)) < 2e-6
     zb = z.to(torch.bfloat16)
     got = o.unary(zb.to(DEV), o.UNARY_GELU)
@@ -159,7 +159,7 @@ def _paged(k, v, P, pages, g, dtype, dc, start=0):
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1.5e-2)])
 @pytest.mark.parametrize("hq,hkv,dk,dv,chunk,P,n,bias,talk", [
-    (6, 3, 8, 8, 21, 8, 75, True, True), (4, 4, 64, 64, 40, 16, 130, True, True), (8, 2, 48, 48, 120, 16, 300, True, True),
+    (6, 3, 8, 8, 21, 8, 75, True, True), (4, 4, 64, 64, 40, 16, 130, True, True), (10, 2, 44, 44, 110, 16, 300, True, True),
     (1, 1, 16, 16, 1, 4, 9, True, True), (16, 1, 8, 8, 1000, 4, 413, True, True), (3, 1, 64, 64, 70, 16, 150, False, True),
     (5, 5, 12, 20, 64, 8, 129, True, False), (16, 4, 64, 64, 256, 16, 600, True, True), (2, 1, 128, 128, 33, 16, 100, True, True),
     (40, 5, 8, 8, 30, 8, 70, True, True), (2, 1, 256, 256, 50, 16, 120, True, True), (12, 12, 36, 36, 90, 16, 200, True, True),
@@ -248,7 +248,7 @@ def test_one_key_that_stands_out_is_found_or_not_seen(dtype, chunk, P, n):
 # ---- attention inside chunks with the framework's attention kernels ------------------------------------------------
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1.5e-2)])
 @pytest.mark.parametrize("hq,hkv,d,chunk,P,n", [(4, 2, 20, 13, 8, 60), (8, 2, 64, 40, 16, 170), (2, 2, 128, 100, 16, 250),
-                                                (16, 1, 16, 1, 4, 11), (8, 2, 128, 120, 16, 400), (4, 4, 64, 64, 16, 257)])
+                                                (16, 1, 16, 1, 4, 11), (6, 2, 128, 112, 16, 400), (4, 4, 64, 64, 16, 257)])
 def test_attention_inside_chunks(dtype, tol, hq, hkv, d, chunk, P, n):
     o = ops()
     g = torch.Generator().manual_seed(chunk + n)
@@ -277,7 +277,7 @@ def test_attention_inside_chunks(dtype, tol, hq, hkv, d, chunk, P, n):
 
 # ---- blends with the token before -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-6), (torch.bfloat16, 8e-3)])
-@pytest.mark.parametrize("W", [80, 192, 1030])
+@pytest.mark.parametrize("W", [80, 208, 1030])
 def test_blends_with_the_token_before_across_cuts_and_slots(dtype, tol, W):
     o = ops()
     g = torch.Generator().manual_seed(W)
@@ -352,7 +352,7 @@ def _run_recurrence(call, inputs, widths, slot, out_cols):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-5)])
-@pytest.mark.parametrize("H,D,Dv,decay", [(2, 12, 8, (0.5, 0.93)), (4, 32, 64, (0.6, 0.88, 0.97, 0.999)), (2, 64, 128, (0.8, 0.99)),
+@pytest.mark.parametrize("H,D,Dv,decay", [(2, 12, 8, (0.5, 0.93)), (4, 24, 48, (0.55, 0.8, 0.95, 0.995)), (2, 64, 128, (0.8, 0.99)),
                                           (3, 4, 20, (1.0, 0.5, 0.25)), (1, 16, 16, (1.0,)), (2, 128, 128, (0.0, 0.9)),
                                           (1, 24, 200, (0.95,))])
 @pytest.mark.parametrize("chunked", [False, True])
@@ -383,7 +383,7 @@ def test_recurrence_with_a_decay_per_head_across_cuts_and_slots(dtype, tol, H, D
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-5)])
-@pytest.mark.parametrize("H,D", [(3, 8), (2, 32), (2, 64), (1, 16), (5, 64), (1, 128), (2, 20)])
+@pytest.mark.parametrize("H,D", [(3, 8), (2, 36), (2, 64), (1, 16), (5, 64), (1, 128), (2, 20)])
 @pytest.mark.parametrize("chunked", [False, True])
 def test_recurrence_with_a_decay_per_channel_and_a_bonus_across_cuts_and_slots(dtype, tol, H, D, chunked):
     o = ops()
