@@ -214,6 +214,26 @@ def test_the_first_tokens_of_a_sequence(tmp_path):
             assert bad is None, f"{first['type']} first, {cut}: {bad}"
 
 
+@pytest.mark.parametrize("kind", ["wkv", "attention", "parallel"])
+def test_models_of_one_kind_of_layer(tmp_path, kind):
+    """Nothing but recurrences (no keys are cached at all), nothing but attention (no state), nothing but the two
+    side by side: two layers each, in every cutting."""
+    layer = {"wkv": wkv(2, 12, ff(40)), "attention": attention(4, 2, 12, 20, 13, 4, 0.3, True, 1000.0, ff(48)),
+             "parallel": parallel(6, 3, 8, 21, 0.35, 30, 2, 12, 8, (0.5, 0.93), 0.7, 1.3, None)}[kind]
+    cfg = dict(PA, layers=[layer, layer])
+    sizes = {0: 7, 1: 7} if kind == "wkv" else {0: 10, 1: 10}
+    folder = write_folder(str(tmp_path / "model"), cfg, random_tensors(cfg, 77, torch.float32, sizes))
+    cfg_, w_ = N.read_folder(folder)
+    reqs = _requests(cfg["vocab"], (50, 3, 29), seed=6)
+    ref = {rid: N.forward(cfg_, w_, toks).float() for rid, toks in reqs.items()}
+    for cut in ("whole", "mixed", "ones"):
+        trace = CUTS[cut](reqs)
+        out = str(tmp_path / cut)
+        traces.run_in_process(trace, folder, "float32", out, 8)
+        bad, worst = traces.first_mismatch(traces.collect(trace, out, cfg["vocab"]), ref, 2e-4)
+        assert bad is None, f"{cut}: first wrong logits at (request, position, relative error) {bad}"
+
+
 # ---- slots and pages -----------------------------------------------------------------------------------------------
 def test_slots_and_pages_that_come_back_start_clean(folders):
     """A request that takes over the state slot and the pages of one that ended computes what it computes alone: the
