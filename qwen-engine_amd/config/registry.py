@@ -93,3 +93,11 @@ def _potatar(d, shapes=None):
 
 
 register_architecture("Potatar", _potatar, tensor_shapes=True)
+
+
+def _safurax(d):
+    from .safurax import SafuraxConfig
+    return SafuraxConfig.from_dict(d)
+
+
+register_architecture("Safurax", _safurax)

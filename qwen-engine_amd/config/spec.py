@@ -57,9 +57,10 @@ class AttentionSpec:
 
 @dataclass(frozen=True)
 class SwiGLUSpec:
-    """down(silu(gate(x)) * up(x)), no biases."""
+    """down(silu(gate(x)) * up(x)), no biases.  ``names``: the tensors of gate, up and down inside the part."""
     intermediate_size: int
     kind: str = "swiglu"
+    names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
 
 
 @dataclass(frozen=True)
@@ -93,7 +94,15 @@ class LatentAttentionSpec:
     query has ``head_dim`` unrotated and ``rot_dim`` rotated numbers, its value ``v_head_dim``.
 
     ``q_rank`` None: queries straight from the input; else through a normed latent of that size.
-    ``output_gate``: the heads' outputs are multiplied by sigmoid of a projection of the mixer's input.
+    ``output_gate``: the heads' outputs are multiplied by sigmoid of a projection of the mixer's input, a number
+    per output, or, with ``gate_per_head``, one number per head.
+    ``window`` None: all earlier keys; else the last ``window`` keys, the query's own included.  ``keep_window``:
+    how many keys the layer's cache keeps where that is more than its own window (a later layer that reads this
+    cache looks further back); None with a window: the window.
+    ``own_latent`` False: the layer has no latent projection; it reads the cache of the layer that the schedule names.
+    ``sink``: a learned number per head whose exponential joins the softmax's denominator and carries no value.
+    ``position``: a rotation of neighbouring pairs (``RopePairsSpec``) or of half-split pairs
+    (``RopeHalfAnglesSpec``) over the first numbers of the rotated part.
     """
     num_heads: int
     head_dim: int
@@ -106,6 +115,11 @@ class LatentAttentionSpec:
     output_gate: bool = False
     position: Optional[object] = None
     kind: str = "latent_attention"
+    gate_per_head: bool = False
+    window: Optional[int] = None
+    keep_window: Optional[int] = None
+    sink: bool = False
+    own_latent: bool = True
 
 
 @dataclass(frozen=True)
@@ -154,10 +168,12 @@ class PostNormLayerSpec:
 class RopeHalfAnglesSpec:
     """Half-split rotation of the first ``rotary_dim`` numbers of a head (number i < rotary_dim / 2 pairs with
     i + rotary_dim / 2) by ``position * theta ** (-2 i / rotary_dim)``; the rest of the head passes unchanged.
-    The kernels form angle, sine and cosine in 32-bit from the frequencies: no table, no limit of positions."""
+    The kernels form angle, sine and cosine in 32-bit from the frequencies: no table, no limit of positions.
+    ``scaling_factor``: every frequency is divided by it (positions stretched linearly)."""
     theta: float
     rotary_dim: int
     kind: str = "rope_half_angles"
+    scaling_factor: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -325,8 +341,59 @@ class LogitSoftcapSpec:
 
 
 @dataclass(frozen=True)
+class BareLayerNormSpec:
+    """y = (x - mean(x)) * rsqrt(mean((x - mean(x))^2) + eps) * w over the last dimension, no bias; the weight tensor
+    carries the part's own name."""
+    eps: float
+    kind: str = "layernorm_bare"
+
+
+@dataclass(frozen=True)
+class DiffAttentionSpec:
+    """Differential attention over grouped heads: every query head and every key head has two maps of ``head_dim``
+    numbers, laid out [map 1 | map 2] in the projections; both maps of a head attend (causally, plain softmax) over
+    the same values of ``v_head_dim`` numbers, and the head's output is a1 - lambda a2, divided by its root mean square
+    (``norm_eps`` inside the root, no weight) and multiplied by 1 - ``diff``.  lambda = exp(lq1 . lk1) - exp(lq2 . lk2)
+    + ``diff`` from four tensors of ``head_dim`` numbers.  ``qk_norm_eps`` not None: every map of every q and k head is
+    RMS-normed with one weight of ``head_dim`` numbers for q and one for k, before the rotation, which turns the
+    first numbers of every map (``position``).  ``output_gate``: a head's output times sigmoid of one number per head,
+    a projection of the mixer's input.  ``names``: the tensors of q, k, v, the output projection and the gate; the
+    norm weights are the projections' names + ``norm_suffix``; the four lambda tensors ``lambda_names``."""
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    scale: float
+    diff: float
+    norm_eps: float
+    qk_norm_eps: Optional[float] = None
+    output_gate: bool = False
+    position: Optional[object] = None
+    names: Tuple[str, str, str, str, str] = ("q", "k", "v", "o", "g")
+    norm_suffix: str = ".norm"
+    lambda_names: Tuple[str, str, str, str] = ("lq1", "lk1", "lq2", "lk2")
+    kind: str = "diff_attention"
+
+
+@dataclass(frozen=True)
+class TopSoftmaxMoESpec:
+    """A routed mixture of small gated feed-forwards down(silu(gate x) * up x) without biases.  The router's 32-bit
+    logits (plus a bias tensor if ``router_bias``) choose the ``top`` largest; their weights are the softmax over the
+    chosen logits alone.  ``shared_intermediate_size``: one more expert of that width that every token uses, added
+    with the weight sigmoid(w_sg . x) if ``shared_gate``, else 1."""
+    num_experts: int
+    top: int
+    intermediate_size: int
+    router_bias: bool = False
+    shared_intermediate_size: Optional[int] = None
+    shared_gate: bool = False
+    kind: str = "top_softmax_moe"
+
+
+@dataclass(frozen=True)
 class LayerSpec:
-    """One pre-norm residual block: x += mixer(norm(x)); x += ffn(norm(x)).
+    """One pre-norm residual block: x += mixer(norm(x)); x += ffn(norm(x)).  ``ffn`` None: the layer is its mixer alone
+    (its second norm is then used only if ``ffn_norm`` is given and the folder holds its tensors).
 
     ``prefix`` is the checkpoint name prefix of the layer's tensors
     (for instance ``model.layers.3``).

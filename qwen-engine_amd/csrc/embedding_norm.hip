@@ -37,18 +37,29 @@ extern "C" int qe_embedding(const int* ids, const void* table, float* out, int T
 template <typename TA, typename TD>
 __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_delta, long delta_stride,
                                const int* __restrict__ rows, const float* __restrict__ w,
-                               TA* __restrict__ out, int H, float eps) {
+                               TA* __restrict__ out, int H, float eps, int center) {
     __shared__ float red[16];
     const long r = blockIdx.x;
     const long src = rows ? (long)rows[r] : r;
     float* hr = h + src * H;
     const TD* dr = delta ? delta + src * H : nullptr;
+    float mean = 0.f;
+    if (center) {                          // (a layer norm: the mean first, then the mean of the squared deviations)
+        float sm = 0.f;
+        for (int c = threadIdx.x; c < H; c += blockDim.x) {
+            float v = hr[c];
+            if (dr)
+                for (int s = 0; s < n_delta; ++s) v += Elem<TD>::load(dr + s * delta_stride + c);
+            sm += v;
+        }
+        mean = block_sum(sm, red) / (float)H;
+    }
     float ss = 0.f;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = hr[c];
         if (dr)
             for (int s = 0; s < n_delta; ++s) v += Elem<TD>::load(dr + s * delta_stride + c);
-        ss += v * v;
+        ss += (v - mean) * (v - mean);
     }
     ss = block_sum(ss, red);
     const float rstd = rsqrtf(ss / (float)H + eps);
@@ -59,7 +70,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ del
         if (dr)
             for (int s = 0; s < n_delta; ++s) v += Elem<TD>::load(dr + s * delta_stride + c);
         if (write_back) hr[c] = v;
-        Elem<TA>::store(o + c, v * rstd * w[c]);
+        Elem<TA>::store(o + c, (v - mean) * rstd * w[c]);
     }
 }
 
@@ -75,7 +86,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ del
 template <typename TA, typename TD, int NV, bool FEW>
 __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_delta, long delta_stride,
                                     const int* __restrict__ rows, const float* __restrict__ w,
-                                    TA* __restrict__ out, int H, float eps) {
+                                    TA* __restrict__ out, int H, float eps, int center) {
     constexpr int SB = !FEW ? 2 : (NV <= 4 ? 8 : 4);
     __shared__ float red[16];
     const long r = blockIdx.x;
@@ -115,12 +126,23 @@ __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ h
     float wv[NV][4];                       // the weights are asked for before the sum is waited for
 #pragma unroll
     for (int i = 0; i < NV; ++i) Vec4<float>::load(w + cs[i], wv[i]);
+    float mean = 0.f;
+    if (center) {                          // (a layer norm: the mean first, then the mean of the squared deviations)
+        float sm = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            if (ok[i]) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sm += v[i][e];
+            }
+        mean = block_sum(sm, red) / (float)H;
+    }
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
         if (ok[i]) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
+            for (int e = 0; e < 4; ++e) ss += (v[i][e] - mean) * (v[i][e] - mean);
         }
     ss = block_sum(ss, red);
     const float rstd = rsqrtf(ss / (float)H + eps);
@@ -132,7 +154,7 @@ __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ h
             if (write_back) Vec4<float>::store(hr + c, v[i]);
             float o[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = v[i][e] * rstd * wv[i][e];
+            for (int e = 0; e < 4; ++e) o[e] = (v[i][e] - mean) * rstd * wv[i][e];
             Vec4<TA>::store(out + r * H + c, o);
         }
     }
@@ -140,7 +162,7 @@ __global__ __launch_bounds__(256) void rmsnorm_regs_kernel(float* __restrict__ h
 
 template <typename TA, typename TD>
 static void launch_rmsnorm(float* h, const void* delta, int n_delta, long stride, const int* rows, const float* w,
-                           void* out, int n_out_rows, int H, float eps, hipStream_t stream) {
+                           void* out, int n_out_rows, int H, float eps, int center, hipStream_t stream) {
     if (H % 4 == 0 && H <= 8192) {
         int threads = ((H / 4 + 63) / 64) * 64;
         if (threads > 256) threads = 256;
@@ -149,10 +171,10 @@ static void launch_rmsnorm(float* h, const void* delta, int n_delta, long stride
     do {                                                                                                     \
         if (n_out_rows <= 512)                                                                               \
             rmsnorm_regs_kernel<TA, TD, NV_, true><<<n_out_rows, threads, 0, stream>>>(                      \
-                h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps);                            \
+                h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps, center);                       \
         else                                                                                                 \
             rmsnorm_regs_kernel<TA, TD, NV_, false><<<n_out_rows, threads, 0, stream>>>(                     \
-                h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps);                            \
+                h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps, center);                       \
     } while (0)
         if (nv <= 1) QE_NORM(1);
         else if (nv <= 2) QE_NORM(2);
@@ -162,23 +184,23 @@ static void launch_rmsnorm(float* h, const void* delta, int n_delta, long stride
         return;
     }
     const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
-    rmsnorm_kernel<TA, TD><<<n_out_rows, threads, 0, stream>>>(h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps);
+    rmsnorm_kernel<TA, TD><<<n_out_rows, threads, 0, stream>>>(h, (const TD*)delta, n_delta, stride, rows, w, (TA*)out, H, eps, center);
 }
 
 // dt_d: element type of delta (that of the output, or float for partial products)
 extern "C" int qe_rmsnorm(float* h, const void* delta, int n_delta, int dt_d, long n_rows_h, const int* rows,
                           const float* w, void* out, int n_out_rows, int H, float eps, int dt_a,
-                          hipStream_t stream) {
+                          int center, hipStream_t stream) {
     QE_REQUIRE(n_out_rows >= 0 && H > 0, "rmsnorm: bad sizes rows=%d H=%d", n_out_rows, H);
     QE_REQUIRE(!delta || n_delta >= 1, "rmsnorm: %d delta tensors", n_delta);
     if (n_out_rows == 0) return 0;
     const long stride = n_rows_h * H;
     if (dt_a == QE_F32 && (!delta || dt_d == QE_F32))
-        launch_rmsnorm<float, float>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, stream);
+        launch_rmsnorm<float, float>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, center, stream);
     else if (dt_a == QE_BF16 && (!delta || dt_d == QE_BF16))
-        launch_rmsnorm<bf16_t, bf16_t>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, stream);
+        launch_rmsnorm<bf16_t, bf16_t>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, center, stream);
     else if (dt_a == QE_BF16 && dt_d == QE_F32)
-        launch_rmsnorm<bf16_t, float>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, stream);
+        launch_rmsnorm<bf16_t, float>(h, delta, n_delta, stride, rows, w, out, n_out_rows, H, eps, center, stream);
     else
         QE_REQUIRE(false, "rmsnorm: no kernel for output type %d with delta type %d", dt_a, dt_d);
     QE_LAUNCH_CHECK();

@@ -1,8 +1,9 @@
 // A matrix product per head: out[t, h, :] = W_h x[t, h, :], W [H, N, K], for all heads in one launch.
 // x and out are addressed with a row and a head stride of their own (in elements), so the product can
 // read a part of each head of a wider tensor and write into a part of each head of another (the
-// unrotated part of the queries into the packed queries).  With ``gate`` ([T, H * N], the activation
-// type) the result is multiplied by sigmoid(gate) before it is stored.
+// unrotated part of the queries into the packed queries).  With ``gate`` (the activation type; the
+// number for token t, head h, output n at gate[t gs_t + h gs_h + n gs_n]: a number per output, or, with gs_n = 0,
+// one per head) the result is multiplied by sigmoid(gate) before it is stored.
 //
 // Any sizes, every multiply-add in IEEE 32-bit, each output summed over k in ascending order whatever
 // T is.  64x64 output tile per block of 256 threads, 4x4 outputs per thread, K in steps of 16 through
@@ -15,7 +16,7 @@
 template <typename TA, typename TW>
 __global__ __launch_bounds__(256) void gemm_heads_kernel(
     const TA* __restrict__ x, long xs_t, long xs_h, const TW* __restrict__ w, TA* __restrict__ out, long os_t,
-    long os_h, const TA* __restrict__ gate, int T, int N, int K) {
+    long os_h, const TA* __restrict__ gate, long gs_t, long gs_h, long gs_n, int T, int N, int K) {
     __shared__ float xs[HK][HT + 4];
     __shared__ float ws[HK][HT + 4];
     const int tid = threadIdx.x;
@@ -65,7 +66,7 @@ __global__ __launch_bounds__(256) void gemm_heads_kernel(
             if (n >= N) continue;
             float v = acc[i][j];
             if (gate) {
-                const float g = Elem<TA>::load(gate + ((long)m * H + h) * N + n);
+                const float g = Elem<TA>::load(gate + (long)m * gs_t + h * gs_h + n * gs_n);
                 v = v / (1.f + expf(-g));
             }
             Elem<TA>::store(out + (long)m * os_t + h * os_h + n, v);
@@ -74,12 +75,13 @@ __global__ __launch_bounds__(256) void gemm_heads_kernel(
 }
 
 extern "C" int qe_gemm_heads(const void* x, long xs_t, long xs_h, const void* w, void* out, long os_t, long os_h,
-                             const void* gate, int T, int H, int N, int K, int dt_a, int dt_w, hipStream_t stream) {
+                             const void* gate, long gs_t, long gs_h, long gs_n, int T, int H, int N, int K, int dt_a,
+                             int dt_w, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && H > 0 && N > 0 && K > 0, "gemm_heads: bad sizes T=%d H=%d N=%d K=%d", T, H, N, K);
     QE_REQUIRE(H <= 65535 && qe_cdiv(T, HT) <= 65535, "gemm_heads: too many heads or rows for one launch");
     if (T == 0) return 0;
     dim3 grid(qe_cdiv(N, HT), qe_cdiv(T, HT), H);
-#define QE_GH(TA_, TW_) gemm_heads_kernel<TA_, TW_><<<grid, 256, 0, stream>>>((const TA_*)x, xs_t, xs_h, (const TW_*)w, (TA_*)out, os_t, os_h, (const TA_*)gate, T, N, K)
+#define QE_GH(TA_, TW_) gemm_heads_kernel<TA_, TW_><<<grid, 256, 0, stream>>>((const TA_*)x, xs_t, xs_h, (const TW_*)w, (TA_*)out, os_t, os_h, (const TA_*)gate, gs_t, gs_h, gs_n, T, N, K)
     if (dt_a == QE_F32 && dt_w == QE_F32) QE_GH(float, float);
     else if (dt_a == QE_BF16 && dt_w == QE_BF16) QE_GH(bf16_t, bf16_t);
     else if (dt_a == QE_BF16 && dt_w == QE_F32) QE_GH(bf16_t, float);
@@ -99,7 +101,7 @@ typedef __attribute__((ext_vector_type(4))) float gh_floatx4;
 template <int MT, int NT>
 __global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(
     const bf16_t* __restrict__ x, long xs_t, long xs_h, const bf16_t* __restrict__ w, bf16_t* __restrict__ out, long os_t,
-    long os_h, const bf16_t* __restrict__ gate, int T, int N, int K) {
+    long os_h, const bf16_t* __restrict__ gate, long gs_t, long gs_h, long gs_n, int T, int N, int K) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, nn = lane & 15;
     const int h = blockIdx.z, H = gridDim.z;
     const int n_base = blockIdx.x * 64 * NT + wave * 16 * NT;      // a wave takes NT groups of 16 features
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(
                 if (n0 + e >= N) break;
                 float v = acc[j][i][e];
                 if (gate) {
-                    const float gv = Elem<bf16_t>::load(gate + ((long)t * H + h) * N + n0 + e);
+                    const float gv = Elem<bf16_t>::load(gate + (long)t * gs_t + h * gs_h + (n0 + e) * gs_n);
                     v = v / (1.f + __expf(-gv));
                 }
                 Elem<bf16_t>::store(o + e, v);
@@ -162,20 +164,21 @@ __global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(
 extern "C" int qe_gemm_heads_mfma_supported(int K, long xs_t, long xs_h) { return K > 0 && K % 8 == 0 && xs_t % 8 == 0 && xs_h % 8 == 0; }
 
 extern "C" int qe_gemm_heads_mfma(const void* x, long xs_t, long xs_h, const void* w, void* out, long os_t, long os_h,
-                                  const void* gate, int T, int H, int N, int K, hipStream_t stream) {
+                                  const void* gate, long gs_t, long gs_h, long gs_n, int T, int H, int N, int K,
+                                  hipStream_t stream) {
     QE_REQUIRE(T >= 0 && H > 0 && N > 0 && qe_gemm_heads_mfma_supported(K, xs_t, xs_h), "gemm_heads (mfma): sizes not taken");
     QE_REQUIRE(H <= 65535, "gemm_heads (mfma): too many heads");
     if (T == 0) return 0;
     if (T <= 32) {
         dim3 grid(qe_cdiv(N, 64), qe_cdiv(T, 16), H);
         gemm_heads_mfma_kernel<1, 1><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
-                                                             os_t, os_h, (const bf16_t*)gate, T, N, K);
+                                                             os_t, os_h, (const bf16_t*)gate, gs_t, gs_h, gs_n, T, N, K);
     } else {
         QE_REQUIRE(qe_cdiv(T, 64) <= 65535, "gemm_heads (mfma): too many rows");
         // (many rows: a wave takes 32 features for 64 tokens, six loads for eight products)
         dim3 grid(qe_cdiv(N, 128), qe_cdiv(T, 64), H);
         gemm_heads_mfma_kernel<4, 2><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
-                                                             os_t, os_h, (const bf16_t*)gate, T, N, K);
+                                                             os_t, os_h, (const bf16_t*)gate, gs_t, gs_h, gs_n, T, N, K);
     }
     QE_LAUNCH_CHECK();
     return 0;

@@ -17,8 +17,11 @@
 //   qe_latent_attention  softmax(scale * q . rows) . rows[:R] per (token, head) over the request's
 //                        positions 0 .. p, 32-bit throughout, any sizes
 //
-// The rotation turns the pair (2i, 2i + 1), i < dims / 2, by position * inv_freq[i]; the angle, its
-// sine and cosine are 32-bit.
+// The rotation turns the pair (2i, 2i + 1), i < dims / 2, by position * inv_freq[i], or, half-split, the pair
+// (i, i + dims / 2); the angle, its sine and cosine are 32-bit.
+//
+// A window of W keys (a token at position p sees the positions p - W + 1 .. p) and a sink (one number a head that
+// joins the softmax's denominator and carries no value) are parameters of the attention kernels.
 #include "common.h"
 
 #define LAT_MAX_R 2048
@@ -31,13 +34,28 @@ __device__ __forceinline__ void turn_pair(float angle, float& u, float& v) {
     v = b;
 }
 
+// Item i of ceil(Dr / 2) handles the numbers a and b (b may lie beyond Dr) and turns them or not.
+__device__ __forceinline__ void pair_place(int i, int rot_dims, int half_split, int& a, int& b, bool& turn) {
+    const int hr = rot_dims >> 1;
+    if (half_split && i < hr) {
+        a = i;
+        b = i + hr;
+        turn = true;
+    } else {
+        a = 2 * i;
+        b = 2 * i + 1;
+        turn = !half_split && b < rot_dims;
+    }
+}
+
 // q (may be null) [T, H, Dn + Dr] -> qp [T, H, R + Dr]: in the same launch, the rotated parts of the token's
 // queries go to the packed queries (what qe_latent_q_rotate does), so that a step of few rows has a kernel less.
 template <typename TC>
 __global__ void latent_kv_store_kernel(const float* __restrict__ kv, const float* __restrict__ weight, float eps,
                                        const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                        int rot_dims, const int* __restrict__ slots, TC* __restrict__ cache,
-                                       int R, int Dr, const TC* __restrict__ q, TC* __restrict__ qp, int H, int Dn) {
+                                       int R, int Dr, const TC* __restrict__ q, TC* __restrict__ qp, int H, int Dn,
+                                       int half_split) {
     __shared__ float red[16];
     const long t = blockIdx.x;
     if (q) {
@@ -47,14 +65,17 @@ __global__ void latent_kv_store_kernel(const float* __restrict__ kv, const float
             const int h = idx / pairs, i = idx % pairs;
             const TC* src = q + (t * H + h) * (Dn + Dr) + Dn;
             TC* dst = qp + (t * H + h) * (R + Dr) + R;
-            if (2 * i + 1 >= Dr) {
-                Elem<TC>::store(dst + 2 * i, Elem<TC>::load(src + 2 * i));
+            int a, b;
+            bool turn;
+            pair_place(i, rot_dims, half_split, a, b, turn);
+            if (b >= Dr) {
+                Elem<TC>::store(dst + a, Elem<TC>::load(src + a));
                 continue;
             }
-            float u = Elem<TC>::load(src + 2 * i), v = Elem<TC>::load(src + 2 * i + 1);
-            if (2 * i + 1 < rot_dims) turn_pair(pq * inv_freq[i], u, v);
-            Elem<TC>::store(dst + 2 * i, u);
-            Elem<TC>::store(dst + 2 * i + 1, v);
+            float u = Elem<TC>::load(src + a), v = Elem<TC>::load(src + b);
+            if (turn) turn_pair(pq * inv_freq[i], u, v);
+            Elem<TC>::store(dst + a, u);
+            Elem<TC>::store(dst + b, v);
         }
     }
     const float* row = kv + t * (R + Dr);
@@ -67,18 +88,25 @@ __global__ void latent_kv_store_kernel(const float* __restrict__ kv, const float
     TC* dst = cache + (long)slot * (R + Dr);
     for (int i = threadIdx.x; i < R; i += blockDim.x) Elem<TC>::store(dst + i, row[i] * f * weight[i]);
     const float p = (float)positions[t];
-    for (int i = threadIdx.x; i < Dr / 2; i += blockDim.x) {
-        float u = row[R + 2 * i], v = row[R + 2 * i + 1];
-        if (2 * i + 1 < rot_dims) turn_pair(p * inv_freq[i], u, v);
-        Elem<TC>::store(dst + R + 2 * i, u);
-        Elem<TC>::store(dst + R + 2 * i + 1, v);
+    for (int i = threadIdx.x; i < (Dr + 1) / 2; i += blockDim.x) {
+        int a, b;
+        bool turn;
+        pair_place(i, rot_dims, half_split, a, b, turn);
+        if (b >= Dr) {                                                 // an odd last number passes
+            Elem<TC>::store(dst + R + a, row[R + a]);
+            continue;
+        }
+        float u = row[R + a], v = row[R + b];
+        if (turn) turn_pair(p * inv_freq[i], u, v);
+        Elem<TC>::store(dst + R + a, u);
+        Elem<TC>::store(dst + R + b, v);
     }
-    if ((Dr & 1) && threadIdx.x == 0) Elem<TC>::store(dst + R + Dr - 1, row[R + Dr - 1]);
 }
 
 extern "C" int qe_latent_kv_store(const float* kv, const float* weight, float eps, const int* positions,
                                   const float* inv_freq, int rot_dims, const int* slots, void* cache, int dt_c,
-                                  int T, int R, int Dr, const void* q, void* qp, int H, int Dn, hipStream_t stream) {
+                                  int T, int R, int Dr, const void* q, void* qp, int H, int Dn, int half_split,
+                                  hipStream_t stream) {
     QE_REQUIRE(!q || (qp && H > 0 && Dn >= 0), "latent_kv_store: queries without a place for them");
     QE_REQUIRE(T >= 0 && R > 0 && Dr >= 0, "latent_kv_store: bad sizes T=%d R=%d Dr=%d", T, R, Dr);
     QE_REQUIRE(rot_dims >= 0 && rot_dims <= Dr && rot_dims % 2 == 0, "latent_kv_store: %d rotated of %d", rot_dims, Dr);
@@ -86,10 +114,10 @@ extern "C" int qe_latent_kv_store(const float* kv, const float* weight, float ep
     const int threads = R >= 512 ? 256 : 64;
     if (dt_c == QE_F32)
         latent_kv_store_kernel<float><<<T, threads, 0, stream>>>(kv, weight, eps, positions, inv_freq, rot_dims, slots,
-                                                                  (float*)cache, R, Dr, (const float*)q, (float*)qp, H, Dn);
+                                                                  (float*)cache, R, Dr, (const float*)q, (float*)qp, H, Dn, half_split);
     else if (dt_c == QE_BF16)
         latent_kv_store_kernel<bf16_t><<<T, threads, 0, stream>>>(kv, weight, eps, positions, inv_freq, rot_dims, slots,
-                                                                   (bf16_t*)cache, R, Dr, (const bf16_t*)q, (bf16_t*)qp, H, Dn);
+                                                                   (bf16_t*)cache, R, Dr, (const bf16_t*)q, (bf16_t*)qp, H, Dn, half_split);
     else
         QE_REQUIRE(false, "latent_kv_store: unknown cache type %d", dt_c);
     QE_LAUNCH_CHECK();
@@ -101,7 +129,7 @@ extern "C" int qe_latent_kv_store(const float* kv, const float* weight, float ep
 template <typename TA>
 __global__ void latent_q_rotate_kernel(const TA* __restrict__ q, const int* __restrict__ positions,
                                        const float* __restrict__ inv_freq, int rot_dims, TA* __restrict__ qp,
-                                       long n_heads_total, int H, int Dn, int Dr, int R) {
+                                       long n_heads_total, int H, int Dn, int Dr, int R, int half_split) {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;      // (token * H + head) * ceil(Dr / 2) + pair
     const int pairs = (Dr + 1) / 2;
     if (idx >= n_heads_total * pairs) return;
@@ -110,18 +138,21 @@ __global__ void latent_q_rotate_kernel(const TA* __restrict__ q, const int* __re
     const long t = th / H;
     const TA* src = q + th * (Dn + Dr) + Dn;
     TA* dst = qp + th * (R + Dr) + R;
-    if (2 * i + 1 >= Dr) {                                             // an odd last number passes
-        Elem<TA>::store(dst + 2 * i, Elem<TA>::load(src + 2 * i));
+    int a, b;
+    bool turn;
+    pair_place(i, rot_dims, half_split, a, b, turn);
+    if (b >= Dr) {                                                     // an odd last number passes
+        Elem<TA>::store(dst + a, Elem<TA>::load(src + a));
         return;
     }
-    float u = Elem<TA>::load(src + 2 * i), v = Elem<TA>::load(src + 2 * i + 1);
-    if (2 * i + 1 < rot_dims) turn_pair((float)positions[t] * inv_freq[i], u, v);
-    Elem<TA>::store(dst + 2 * i, u);
-    Elem<TA>::store(dst + 2 * i + 1, v);
+    float u = Elem<TA>::load(src + a), v = Elem<TA>::load(src + b);
+    if (turn) turn_pair((float)positions[t] * inv_freq[i], u, v);
+    Elem<TA>::store(dst + a, u);
+    Elem<TA>::store(dst + b, v);
 }
 
 extern "C" int qe_latent_q_rotate(const void* q, const int* positions, const float* inv_freq, int rot_dims, void* qp,
-                                  int dt_a, int T, int H, int Dn, int Dr, int R, hipStream_t stream) {
+                                  int dt_a, int T, int H, int Dn, int Dr, int R, int half_split, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && H > 0 && Dn >= 0 && Dr >= 0 && R > 0, "latent_q_rotate: bad sizes");
     QE_REQUIRE(rot_dims >= 0 && rot_dims <= Dr && rot_dims % 2 == 0, "latent_q_rotate: %d rotated of %d", rot_dims, Dr);
     const long n = (long)T * H * ((Dr + 1) / 2);
@@ -129,24 +160,24 @@ extern "C" int qe_latent_q_rotate(const void* q, const int* positions, const flo
     const int blocks = qe_cdiv(n, 256);
     if (dt_a == QE_F32)
         latent_q_rotate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)q, positions, inv_freq, rot_dims,
-                                                                   (float*)qp, (long)T * H, H, Dn, Dr, R);
+                                                                   (float*)qp, (long)T * H, H, Dn, Dr, R, half_split);
     else if (dt_a == QE_BF16)
         latent_q_rotate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)q, positions, inv_freq, rot_dims,
-                                                                    (bf16_t*)qp, (long)T * H, H, Dn, Dr, R);
+                                                                    (bf16_t*)qp, (long)T * H, H, Dn, Dr, R, half_split);
     else
         QE_REQUIRE(false, "latent_q_rotate: unknown type %d", dt_a);
     QE_LAUNCH_CHECK();
     return 0;
 }
 
-// One wave per (token, head).  Keys are taken 64 at a time from position 0 upwards with an online
-// softmax, so the order of the sums depends on the position only: not on how the request's tokens
-// were cut into steps, nor on what else is in the batch.
+// One wave per (token, head).  Keys are taken 64 at a time from the first position the token sees (0, or
+// p - window + 1) upwards with an online softmax, so the order of the sums depends on the position only: not on
+// how the request's tokens were cut into steps, nor on what else is in the batch.  The sink joins at the end.
 template <typename TA>
 __global__ __launch_bounds__(64) void latent_attention_kernel(
     const TA* __restrict__ qp, TA* __restrict__ out, const TA* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
-    int max_blocks, int H, int R, int Dr, int P, float scale) {
+    int max_blocks, int H, int R, int Dr, int P, float scale, int window, const float* __restrict__ sink) {
     extern __shared__ float smem[];
     const int D = R + Dr;
     float* qs = smem;                                   // D
@@ -166,7 +197,8 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
 #pragma unroll
     for (int i = 0; i < LAT_MAX_R / 64; ++i) acc[i] = 0.f;
 
-    for (int j0 = 0; j0 <= p; j0 += 64) {
+    const int first = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    for (int j0 = first; j0 <= p; j0 += 64) {
         const int j = j0 + lane;
         float sc = -INFINITY;
         long ro = 0;
@@ -197,7 +229,11 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
         }
         __syncthreads();
     }
-    const float inv = 1.f / l;
+    float inv = 1.f / l;
+    if (sink) {                                        // one more entry of score sink[h], with no value
+        const float sk = sink[h], mt = fmaxf(m, sk), f = expf(m - mt);
+        inv = f / (l * f + expf(sk - mt));
+    }
     TA* orow = out + (t * H + h) * R;
 #pragma unroll
     for (int i = 0; i < LAT_MAX_R / 64; ++i) {
@@ -209,7 +245,9 @@ __global__ __launch_bounds__(64) void latent_attention_kernel(
 // qp [T, H, R + Dr] -> out [T, H, R]
 extern "C" int qe_latent_attention(const void* qp, void* out, const void* cache, const int* positions,
                                    const int* tok_seq, const int* block_table, int max_blocks, int T, int H, int R,
-                                   int Dr, int P, float scale, int dt_a, hipStream_t stream) {
+                                   int Dr, int P, float scale, int window, const float* sink, int dt_a,
+                                   hipStream_t stream) {
+    QE_REQUIRE(window >= 0, "latent_attention: a window of %d keys", window);
     QE_REQUIRE(R > 0 && R <= LAT_MAX_R, "latent_attention: latent size %d exceeds %d", R, LAT_MAX_R);
     QE_REQUIRE(H > 0 && H <= 65535 && Dr >= 0 && P > 0, "latent_attention: bad sizes");
     if (T == 0) return 0;
@@ -217,10 +255,10 @@ extern "C" int qe_latent_attention(const void* qp, void* out, const void* cache,
     const size_t shmem = (size_t)((R + Dr + 64 + 1) & ~1) * sizeof(float) + 64 * sizeof(long);
     if (dt_a == QE_F32)
         latent_attention_kernel<float><<<grid, 64, shmem, stream>>>((const float*)qp, (float*)out, (const float*)cache,
-                                                                     positions, tok_seq, block_table, max_blocks, H, R, Dr, P, scale);
+                                                                     positions, tok_seq, block_table, max_blocks, H, R, Dr, P, scale, window, sink);
     else if (dt_a == QE_BF16)
         latent_attention_kernel<bf16_t><<<grid, 64, shmem, stream>>>((const bf16_t*)qp, (bf16_t*)out, (const bf16_t*)cache,
-                                                                      positions, tok_seq, block_table, max_blocks, H, R, Dr, P, scale);
+                                                                      positions, tok_seq, block_table, max_blocks, H, R, Dr, P, scale, window, sink);
     else
         QE_REQUIRE(false, "latent_attention: unknown type %d", dt_a);
     QE_LAUNCH_CHECK();

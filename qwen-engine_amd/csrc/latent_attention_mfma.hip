@@ -21,6 +21,11 @@
 // takes the keys [s L, (s + 1) L), L = ceil((p + 1) / NS) rounded up to 32.  With NS > 1 the splits' partial
 // results (running maximum, sum, unnormalised output, 32-bit) go to a workspace and a second kernel merges
 // them in the order of s.
+//
+// With a window of W keys a token at position p sees the positions p - W + 1 .. p: a token group's walk starts at
+// the first position that its first row sees, and the splits cut what lies between that and the last row's position.
+// With a sink (one number a head) the softmax's denominator has exp(sink) added, at the end of an uncut walk or
+// where the splits are merged.
 #include "attention_tile.h"
 
 // bf16 per row of the transposed tile: 32 keys and 4 of padding, 18 words.  A thread writes eight rows that
@@ -35,7 +40,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ qp, bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
     const bf16_t* __restrict__ cache, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks, int T, int H, int R, int Dk, int P, float scale,
-    int TOK, int HGB, int NS) {
+    int TOK, int HGB, int NS, int window, const float* __restrict__ sink) {
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];
     const int dkc = (Dk + 31) / 32, rb = (R + 15) / 16;
     const int kpitch = dkc * 32 + 8;
@@ -75,11 +80,13 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
         int end = seg + 1;
         while (end < TOK && t0 + end < T && tok_seq[t0 + end] == req) ++end;
         const int kmax = positions[t0 + end - 1];                  // (positions rise within a request's rows)
-        const int L = ((kmax + NS) / NS + 31) & ~31;
-        const int k0 = split * L;
+        const int kfirst = window > 0 ? max(0, positions[t0 + seg] - window + 1) : 0;
+        const int L = ((kmax - kfirst + NS) / NS + 31) & ~31;
+        const int k0 = kfirst + split * L;
         const int k1 = min(k0 + L, kmax + 1);
         const bool mine = unit_ok && wt >= seg && wt < end;
         const int p = mine ? positions[t] : -1;
+        const int plo = window > 0 ? p - window : -1;              // the keys above this position are seen
         const int* bt = block_table + (long)req * max_blocks;
         // The rows' places in the cache for up to LAT_CHUNK keys at a time, so that no load of a tile waits for
         // the block table; a tile's loads are issued before the tile before it is computed and go to shared
@@ -150,8 +157,8 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int ka = kk + g * 4 + j, kb = ka + 16;
-                sv[j] = (ka <= p && ka < k1) ? s0[j] * scale : -INFINITY;
-                sv[4 + j] = (kb <= p && kb < k1) ? s1[j] * scale : -INFINITY;
+                sv[j] = (ka <= p && ka > plo && ka < k1) ? s0[j] * scale : -INFINITY;
+                sv[4 + j] = (kb <= p && kb > plo && kb < k1) ? s1[j] * scale : -INFINITY;
                 tmax = fmaxf(tmax, fmaxf(sv[j], sv[4 + j]));
             }
             tmax = max_over_lane_rows(tmax);
@@ -189,7 +196,11 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
             ls += __shfl_xor(ls, 32, 64);
             if (head_ok) {
                 if (NS == 1) {
-                    const float inv = 1.f / ls;
+                    float inv = 1.f / ls;
+                    if (sink) {
+                        const float sk = sink[head], mt = fmaxf(m, sk), f = __expf(m - mt);
+                        inv = f / (ls * f + __expf(sk - mt));
+                    }
                     bf16_t* o = out + ((long)t * H + head) * R;
 #pragma unroll
                     for (int db = 0; db < RB; ++db) {
@@ -222,7 +233,8 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 // thread adds up its output numbers, eight splits' loads at a time.
 __global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float* __restrict__ part_acc,
                                                                      const float* __restrict__ part_ml,
-                                                                     bf16_t* __restrict__ out, int NS, int R, int RP) {
+                                                                     bf16_t* __restrict__ out, int NS, int R, int RP,
+                                                                     const float* __restrict__ sink, int H) {
     __shared__ float wgt[64];
     __shared__ float inv_l;
     const long th = blockIdx.x;
@@ -231,10 +243,12 @@ __global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float
         const float* pm = part_ml + th * NS * 2;
         const float ms = tid < NS ? pm[2 * tid] : -INFINITY;
         const float ls = tid < NS ? pm[2 * tid + 1] : 0.f;
-        const float M = wave_max(ms);
+        float M = wave_max(ms);
+        const float sk = sink ? sink[th % H] : -INFINITY;
+        M = fmaxf(M, sk);
         const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
         wgt[tid] = w;
-        float L = 0.f;
+        float L = sink ? __expf(sk - M) : 0.f;
         for (int s = 0; s < NS; ++s) L = fmaf(__shfl(w, s, 64), __shfl(ls, s, 64), L);      // in the order of the splits
         if (tid == 0) inv_l = 1.f / L;
     }
@@ -272,7 +286,7 @@ extern "C" int qe_latent_attention_mfma_supported(int R, int Dr) {
 }
 
 // How the step's rows are laid over blocks and the keys over splits: from the shapes alone.
-static void latent_plan(int T, int H, int& TOK, int& HGB, int& NS) {
+static void latent_plan(int T, int H, int window, int& TOK, int& HGB, int& NS) {
     const int HG = (H + 15) / 16;
     HGB = HG < 4 ? HG : 4;
     TOK = T <= 64 ? 1 : (4 / HGB > 1 ? 4 / HGB : 1);
@@ -287,11 +301,15 @@ static void latent_plan(int T, int H, int& TOK, int& HGB, int& NS) {
         if (cap > 32) cap = 32;
         if (NS > cap) NS = cap;
     }
+    if (window > 0) {                // (a walk is no longer than the window and the block's rows: no more splits than tiles)
+        const int tiles = (window + TOK + 30) / 32;
+        if (NS > tiles) NS = tiles;
+    }
 }
 
-extern "C" long qe_latent_attention_mfma_workspace_bytes(int T, int H, int R) {
+extern "C" long qe_latent_attention_mfma_workspace_bytes(int T, int H, int R, int window) {
     int TOK, HGB, NS;
-    latent_plan(T, H, TOK, HGB, NS);
+    latent_plan(T, H, window, TOK, HGB, NS);
     if (NS == 1) return 0;
     const long RP = (long)((R + 15) / 16) * 16;
     return (long)T * H * NS * (RP + 2) * sizeof(float);
@@ -299,18 +317,18 @@ extern "C" long qe_latent_attention_mfma_workspace_bytes(int T, int H, int R) {
 
 extern "C" int qe_latent_attention_mfma(const void* qp, void* out, const void* cache, const int* positions,
                                         const int* tok_seq, const int* block_table, int max_blocks, int T, int H,
-                                        int R, int Dr, int P, float scale, void* workspace, long workspace_bytes,
-                                        hipStream_t stream) {
+                                        int R, int Dr, int P, float scale, int window, const float* sink,
+                                        void* workspace, long workspace_bytes, hipStream_t stream) {
     int rbc, dkcc;
     const int Dk = R + Dr;
     QE_REQUIRE(latent_mfma_fits(R, Dk, rbc, dkcc), "latent_attention (mfma): sizes R=%d Dr=%d not taken", R, Dr);
-    QE_REQUIRE(H > 0 && P > 0, "latent_attention (mfma): bad sizes");
+    QE_REQUIRE(H > 0 && P > 0 && window >= 0, "latent_attention (mfma): bad sizes");
     if (T == 0) return 0;
     int TOK, HGB, NS;
-    latent_plan(T, H, TOK, HGB, NS);
+    latent_plan(T, H, window, TOK, HGB, NS);
     const int HG = (H + 15) / 16;
     const long RP = (long)((R + 15) / 16) * 16;
-    QE_REQUIRE(workspace_bytes >= qe_latent_attention_mfma_workspace_bytes(T, H, R), "latent_attention (mfma): workspace too small");
+    QE_REQUIRE(workspace_bytes >= qe_latent_attention_mfma_workspace_bytes(T, H, R, window), "latent_attention (mfma): workspace too small");
     QE_REQUIRE(NS <= 64 && qe_cdiv(HG, HGB) <= 65535, "latent_attention (mfma): grid too large");
     float* part_acc = (float*)workspace;
     float* part_ml = part_acc ? part_acc + (long)T * H * NS * RP : nullptr;
@@ -329,7 +347,7 @@ extern "C" int qe_latent_attention_mfma(const void* qp, void* out, const void* c
         }                                                                                                             \
         latent_attention_mfma_kernel<RB_, DKC_><<<grid, 256, shmem, stream>>>(                                        \
             (const bf16_t*)qp, (bf16_t*)out, part_acc, part_ml, (const bf16_t*)cache, positions, tok_seq, block_table, \
-            max_blocks, T, H, R, Dk, P, scale, TOK, HGB, NS);                                                         \
+            max_blocks, T, H, R, Dk, P, scale, TOK, HGB, NS, window, sink);                                                       \
     } while (0)
     if (rbc == 4) QE_LA(4, 4);
     else if (rbc == 8) QE_LA(8, 6);
@@ -338,7 +356,7 @@ extern "C" int qe_latent_attention_mfma(const void* qp, void* out, const void* c
 #undef QE_LA
     QE_LAUNCH_CHECK();
     if (NS > 1) {
-        latent_attention_merge_kernel<<<T * H, R >= 256 ? 256 : (R >= 128 ? 128 : 64), 0, stream>>>(part_acc, part_ml, (bf16_t*)out, NS, R, (int)RP);
+        latent_attention_merge_kernel<<<T * H, R >= 256 ? 256 : (R >= 128 ? 128 : 64), 0, stream>>>(part_acc, part_ml, (bf16_t*)out, NS, R, (int)RP, sink, H);
         QE_LAUNCH_CHECK();
     }
     return 0;

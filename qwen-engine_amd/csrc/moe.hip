@@ -108,30 +108,37 @@ extern "C" int qe_moe_route(const float* logits, int* ids, float* weights, int T
 
 
 // One token's routing by one wave: softmax over all E outputs, choice by score + correction, weights from the
-// scores alone.  sc: the wave's own 2 E + top floats of shared memory.  Every wave of the block calls it together
+// scores alone.  Without a correction (null) the choice goes by the logits themselves and the weights are the
+// softmax over the chosen logits alone (the scores stay unnormalised: the largest is 1, so the chosen ones' sum
+// is at least 1 however far the others lie below).  sc: the wave's own 2 E + top floats of shared memory.  Every wave of the block calls it together
 // (the barriers are the block's); a wave without a token (z null) only keeps step.
 __device__ __forceinline__ void route_biased_token(const float* __restrict__ z, const float* __restrict__ correction,
                                                    float* sc, int* __restrict__ ids, float* __restrict__ weights, int E,
-                                                   int top, float scale, int lane, long zs = 1) {
+                                                   int top, float scale, int lane, long zs = 1,
+                                                   const float* __restrict__ zbias = nullptr) {
     float* ch = sc + E;
     float* picked = ch + E;
-    if (z) {                                             // (zs: the distance between a token's logits)
+    if (z) {                                             // (zs: the distance between a token's logits; zbias: added to them)
         float mx = -INFINITY;
-        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e * zs]);
+        for (int e = lane; e < E; e += 64) {
+            const float zv = z[e * zs] + (zbias ? zbias[e] : 0.f);
+            ch[e] = zv;
+            mx = fmaxf(mx, zv);
+        }
         mx = wave_max(mx);
         float sum = 0.f;
         for (int e = lane; e < E; e += 64) {
-            const float ex = expf(z[e * zs] - mx);
+            const float ex = expf(ch[e] - mx);
             sc[e] = ex;
             sum += ex;
         }
         sum = wave_sum(sum);
         for (int e = lane; e < E; e += 64) {
-            float v = sc[e] / sum;
+            float v = correction ? sc[e] / sum : sc[e];
             if (!(v == v)) v = 0.f;            // (a row of garbage still gets experts inside the table)
             sc[e] = v;
-            float c = v + correction[e];
-            if (!(c == c)) c = 0.f;
+            float c = correction ? v + correction[e] : ch[e];
+            if (!(c == c)) c = correction ? 0.f : -3.0e38f;
             ch[e] = c;
         }
     }
@@ -160,20 +167,23 @@ __device__ __forceinline__ void route_biased_token(const float* __restrict__ z, 
 
 __global__ __launch_bounds__(64) void moe_route_biased_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
                                                               int* __restrict__ ids, float* __restrict__ weights, int E, int top,
-                                                              float scale, int transposed) {
+                                                              float scale, int transposed, const float* __restrict__ zbias,
+                                                              int ld) {
     extern __shared__ float sc[];          // E scores, E choice scores, top chosen scores
     const long t = blockIdx.x;
     // (transposed: logits [E, T], as a product of the router's few rows against the tokens' many leaves them)
-    route_biased_token(transposed ? logits + t : logits + t * E, correction, sc, ids + t * top, weights + t * top, E, top,
-                       scale, threadIdx.x, transposed ? (long)gridDim.x : 1L);
+    route_biased_token(transposed ? logits + t : logits + t * ld, correction, sc, ids + t * top, weights + t * top, E, top,
+                       scale, threadIdx.x, transposed ? (long)gridDim.x : 1L, zbias);
 }
 
 extern "C" int qe_moe_route_biased(const float* logits, const float* correction, int* ids, float* weights, int T, int E,
-                                   int top, float scale, int transposed, hipStream_t stream) {
+                                   int top, float scale, int transposed, const float* zbias, int ld, hipStream_t stream) {
+    if (ld <= 0) ld = E;                   // (ld: the distance between two tokens' logits where they are not transposed)
+    QE_REQUIRE(ld >= E, "moe_route_biased: rows of %d logits for %d experts", ld, E);
     QE_REQUIRE(T >= 0 && E > 0 && top >= 1 && top <= E, "moe_route_biased: top %d of %d experts", top, E);
     QE_REQUIRE((2 * E + top) * sizeof(float) <= 60000, "moe_route_biased: too many experts");
     if (T == 0) return 0;
-    moe_route_biased_kernel<<<T, 64, (2 * E + top) * sizeof(float), stream>>>(logits, correction, ids, weights, E, top, scale, transposed);
+    moe_route_biased_kernel<<<T, 64, (2 * E + top) * sizeof(float), stream>>>(logits, correction, ids, weights, E, top, scale, transposed, zbias, ld);
     QE_LAUNCH_CHECK();
     return 0;
 }
@@ -264,7 +274,8 @@ template <typename TA>
 __global__ __launch_bounds__(1024) void moe_front_small_kernel(
     const float* __restrict__ logits, const float* __restrict__ correction, const TA* __restrict__ x, int* __restrict__ ids,
     float* __restrict__ weights, int* __restrict__ perm, int* __restrict__ inv, int* __restrict__ tiles,
-    int* __restrict__ n_tiles, float* __restrict__ parts, int T, int H, int E, int E_real, int top, float scale, int tile_rows) {
+    int* __restrict__ n_tiles, float* __restrict__ parts, int T, int H, int E, int E_real, int top, float scale, int tile_rows,
+    const float* __restrict__ zbias, int ld) {
     extern __shared__ int sm[];
     const int n = T * top;
     int* ids_s = sm;                                     // n
@@ -274,8 +285,8 @@ __global__ __launch_bounds__(1024) void moe_front_small_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     for (int t0 = 0; t0 < T; t0 += waves) {
         const int t = t0 + wave;
-        route_biased_token(t < T ? logits + (long)t * E : nullptr, correction, wave_sc + (long)wave * (2 * E + top),
-                           ids_s + (t < T ? t : 0) * top, w_s + (t < T ? t : 0) * top, E, top, scale, lane);
+        route_biased_token(t < T ? logits + (long)t * ld : nullptr, correction, wave_sc + (long)wave * (2 * E + top),
+                           ids_s + (t < T ? t : 0) * top, w_s + (t < T ? t : 0) * top, E, top, scale, lane, 1L, zbias);
     }
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -304,16 +315,18 @@ extern "C" int qe_moe_front_small_supported(int T, int E, int top) {
 // parts of the pairs that chose an identity expert (E_real .. E - 1) are written, the others left.
 extern "C" int qe_moe_front_small(const float* logits, const float* correction, const void* x, int* ids, float* weights,
                                   int* perm, int* inv, int* tiles, int* n_tiles, float* parts, int max_tiles, int T, int H,
-                                  int E, int E_real, int top, float scale, int tile_rows, int dt_a, hipStream_t stream) {
+                                  int E, int E_real, int top, float scale, int tile_rows, int dt_a, const float* zbias, int ld,
+                                  hipStream_t stream) {
+    if (ld <= 0) ld = E;
     QE_REQUIRE(qe_moe_front_small_supported(T, E, top), "moe_front_small: %d tokens, %d outputs, top %d", T, E, top);
     QE_REQUIRE(E_real >= 1 && E_real <= E && top <= E && tile_rows > 0 && H > 0, "moe_front_small: bad sizes");
     const int n = T * top;
     QE_REQUIRE(max_tiles >= (n + tile_rows - 1) / tile_rows + (E_real < n ? E_real : n), "moe_front_small: %d tiles may not be enough", max_tiles);
     const size_t lds = ((size_t)2 * n + 2 * E + 16 * (2 * E + top)) * 4;
     if (dt_a == QE_BF16)
-        moe_front_small_kernel<bf16_t><<<1, 1024, lds, stream>>>(logits, correction, (const bf16_t*)x, ids, weights, perm, inv, tiles, n_tiles, parts, T, H, E, E_real, top, scale, tile_rows);
+        moe_front_small_kernel<bf16_t><<<1, 1024, lds, stream>>>(logits, correction, (const bf16_t*)x, ids, weights, perm, inv, tiles, n_tiles, parts, T, H, E, E_real, top, scale, tile_rows, zbias, ld);
     else if (dt_a == QE_F32)
-        moe_front_small_kernel<float><<<1, 1024, lds, stream>>>(logits, correction, (const float*)x, ids, weights, perm, inv, tiles, n_tiles, parts, T, H, E, E_real, top, scale, tile_rows);
+        moe_front_small_kernel<float><<<1, 1024, lds, stream>>>(logits, correction, (const float*)x, ids, weights, perm, inv, tiles, n_tiles, parts, T, H, E, E_real, top, scale, tile_rows, zbias, ld);
     else
         QE_REQUIRE(false, "moe_front_small: unknown type %d", dt_a);
     QE_LAUNCH_CHECK();
@@ -415,9 +428,14 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
             for (int j = 0; j < 4; ++j) {
                 const int n = n0 + tx * 4 + j;
                 if (n >= N) continue;
-                const float g = fminf(acc[i][j], limit);
-                const float u = fminf(fmaxf(acu[i][j], -limit), limit);
-                Elem<TA>::store(o + n, g / (1.f + expf(-slope * g)) * (u + 1.f));
+                if (limit > 0.f) {
+                    const float g = fminf(acc[i][j], limit);
+                    const float u = fminf(fmaxf(acu[i][j], -limit), limit);
+                    Elem<TA>::store(o + n, g / (1.f + expf(-slope * g)) * (u + 1.f));
+                } else {                               // (no limit: the plain silu(g) u)
+                    const float g = acc[i][j];
+                    Elem<TA>::store(o + n, g / (1.f + expf(-g)) * acu[i][j]);
+                }
             }
         } else {
             const int pair = perm[r0 + m];
@@ -500,6 +518,34 @@ extern "C" int qe_moe_combine(const void* y, const int* inv, const float* weight
     if (dt_y == QE_F32) moe_combine_kernel<float><<<T, 256, 0, stream>>>((const float*)y, inv, weights, out, top, H);
     else if (dt_y == QE_BF16) moe_combine_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)y, inv, weights, out, top, H);
     else QE_REQUIRE(false, "moe_combine: unknown type %d", dt_y);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+
+// dst[t, :] (+)= sigmoid(s[t * ss]) * src[t, :]: an expert that every token uses, weighed by a gate of one number a
+// token, written as one more part of the mixture's output or added to the sum that is already there.
+template <typename TS>
+__global__ void moe_row_gate_kernel(float* __restrict__ dst, const TS* __restrict__ src, const float* __restrict__ s, long ss,
+                                    int T, int H, int accumulate) {
+    const long n = (long)T * H;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const long t = i / H;
+        const float g = 1.f / (1.f + expf(-s[t * ss]));
+        const float v = g * Elem<TS>::load(src + i);
+        dst[i] = accumulate ? dst[i] + v : v;
+    }
+}
+
+extern "C" int qe_moe_row_gate(float* dst, const void* src, int dt_s, const float* s, long ss, int T, int H, int accumulate,
+                               hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && H > 0 && ss >= 1, "moe_row_gate: bad sizes");
+    if (T == 0) return 0;
+    const long n = (long)T * H;
+    const int blocks = (int)((n + 255) / 256 > 8192 ? 8192 : (n + 255) / 256);
+    if (dt_s == QE_F32) moe_row_gate_kernel<float><<<blocks, 256, 0, stream>>>(dst, (const float*)src, s, ss, T, H, accumulate);
+    else if (dt_s == QE_BF16) moe_row_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(dst, (const bf16_t*)src, s, ss, T, H, accumulate);
+    else QE_REQUIRE(false, "moe_row_gate: unknown element type %d", dt_s);
     QE_LAUNCH_CHECK();
     return 0;
 }

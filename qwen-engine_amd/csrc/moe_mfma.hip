@@ -87,9 +87,14 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if (n0 + j >= N) break;
-                const float gv = fminf(ag[i][j], limit);
-                const float uv = fminf(fmaxf(au[i][j], -limit), limit);
-                Elem<bf16_t>::store(o + j, gv / (1.f + __expf(-slope * gv)) * (uv + 1.f));
+                if (limit > 0.f) {
+                    const float gv = fminf(ag[i][j], limit);
+                    const float uv = fminf(fmaxf(au[i][j], -limit), limit);
+                    Elem<bf16_t>::store(o + j, gv / (1.f + __expf(-slope * gv)) * (uv + 1.f));
+                } else {                               // (no limit: the plain silu(g) u)
+                    const float gv = ag[i][j];
+                    Elem<bf16_t>::store(o + j, gv / (1.f + __expf(-gv)) * au[i][j]);
+                }
             }
         } else {
             const int pair = perm[r0 + m];

@@ -43,7 +43,7 @@ def load_library():
     vp, i32, f32, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
     sigs = {
         "qe_embedding": [vp, vp, vp, i32, i32, i32, i32, vp],
-        "qe_rmsnorm": [vp, vp, i32, i32, i64, vp, vp, vp, i32, i32, f32, i32, vp],
+        "qe_rmsnorm": [vp, vp, i32, i32, i64, vp, vp, vp, i32, i32, f32, i32, i32, vp],
         "qe_residual_add": [vp, vp, i64, i32, vp],
         "qe_scatter_int": [vp, vp, vp, i32, i64, vp],
         "qe_silu_mul": [vp, vp, i32, i32, i32, i32, vp],
@@ -78,9 +78,11 @@ def load_library():
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32, vp],
         "qe_qkv_conv_rope_store": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_scale_f32": [vp, i64, f32, vp],
-        "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, i32, vp],
+        "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, i32, vp, i32, vp],
         "qe_moe_front_small_supported": [i32, i32, i32],
-        "qe_moe_front_small": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, vp],
+        "qe_moe_front_small": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, vp, i32, vp],
+        "qe_moe_row_gate": [vp, vp, i32, vp, i64, i32, i32, i32, vp],
+        "qe_diff_heads": [vp, vp, vp, i64, i32, i32, i32, i32, i32, f32, f32, f32, i32, vp],
         "qe_moe_identity": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_argmax_static": [vp, vp, i32, i32, vp],
@@ -102,14 +104,14 @@ def load_library():
         "qe_scaled_sum": [vp, f32, vp, f32, i32, vp, i64, vp],
         "qe_polynorm": [vp, vp, f32, vp, i32, i32, i32, vp],
         "qe_short_conv": [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
-        "qe_latent_kv_store": [vp, vp, f32, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, i32, i32, vp],
-        "qe_latent_q_rotate": [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, vp],
-        "qe_latent_attention": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp],
+        "qe_latent_kv_store": [vp, vp, f32, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, i32, i32, i32, vp],
+        "qe_latent_q_rotate": [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_latent_attention": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp, i32, vp],
         "qe_latent_attention_mfma_supported": [i32, i32],
-        "qe_latent_attention_mfma": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, vp, i64, vp],
-        "qe_gemm_heads": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32, vp],
+        "qe_latent_attention_mfma": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp, vp, i64, vp],
+        "qe_gemm_heads": [vp, i64, i64, vp, vp, i64, i64, vp, i64, i64, i64, i32, i32, i32, i32, i32, i32, vp],
         "qe_gemm_heads_mfma_supported": [i32, i64, i64],
-        "qe_gemm_heads_mfma": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, vp],
+        "qe_gemm_heads_mfma": [vp, i64, i64, vp, vp, i64, i64, vp, i64, i64, i64, i32, i32, i32, i32, vp],
         "qe_moe_route": [vp, vp, vp, i32, i32, i32, i32, i32, vp],
         "qe_moe_sort": [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32, vp],
         "qe_moe_gemm": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, i32, i32, i32, vp],
@@ -136,7 +138,7 @@ def load_library():
     lib.qe_attention_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
     lib.qe_attention_decode_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_prefill_workspace_bytes.restype = ctypes.c_long
-    lib.qe_latent_attention_mfma_workspace_bytes.argtypes = [i32, i32, i32]
+    lib.qe_latent_attention_mfma_workspace_bytes.argtypes = [i32, i32, i32, i32]
     lib.qe_latent_attention_mfma_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_prefill_workspace_bytes_for.restype = ctypes.c_long
     _lib = lib
@@ -220,8 +222,9 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor
 
 def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
-            out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """RMSNorm of the 32-bit stream h [T, H] into out_dtype.
+            out: Optional[torch.Tensor] = None, center: bool = False) -> torch.Tensor:
+    """RMSNorm of the 32-bit stream h [T, H] into out_dtype; with ``center`` a layer norm without bias:
+    (v - mean) * rsqrt(mean of the squared deviations + eps) * weight.
 
     With ``delta`` the residual sum h + delta is normed; it is written back to h
     unless ``rows`` is given.  delta is [T, H] in out_dtype, or float32 [S, T, H]:
@@ -248,7 +251,7 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
         out = torch.empty((n, H), dtype=out_dtype, device=h.device)
     _need(out, "out", out_dtype, (n, H), h.device)
     _check(lib.qe_rmsnorm(h.data_ptr(), _ptr(delta), n_delta, dt_d, T, _ptr(rows), weight.data_ptr(),
-                          out.data_ptr(), n, H, float(eps), _DT[out_dtype], _stream()), "rmsnorm")
+                          out.data_ptr(), n, H, float(eps), _DT[out_dtype], int(bool(center)), _stream()), "rmsnorm")
     return out
 
 
@@ -948,9 +951,11 @@ def short_conv(x: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], 
 # ---- attention over one cached latent per token --------------------------------------------------------
 def latent_kv_store(kv: torch.Tensor, weight: torch.Tensor, eps: float, positions: torch.Tensor,
                     inv_freq: torch.Tensor, slots: Optional[torch.Tensor], cache: torch.Tensor,
-                    q: Optional[torch.Tensor] = None, qp: Optional[torch.Tensor] = None, dim: int = 0) -> None:
+                    q: Optional[torch.Tensor] = None, qp: Optional[torch.Tensor] = None, dim: int = 0,
+                    half_split: bool = False) -> None:
     """kv float32 [T, R + Dr] (R = weight's length): the first R normed (weight * u / rms(u)), the last Dr
-    turned in neighbouring pairs by positions * inv_freq (float32 [n], 2 n <= Dr; the rest passes), into
+    turned in neighbouring pairs (``half_split``: number i with number i + n) by positions * inv_freq (float32 [n],
+    2 n <= Dr; the rest passes), into
     the row slots[t] of cache [pages, 1, 1, P, R + Dr] (negative slot, or no slots: nowhere).  With q
     [T, H, dim + Dr] and qp [T, H, R + Dr] the same launch does what latent_q_rotate does."""
     lib = load_library()
@@ -971,11 +976,12 @@ def latent_kv_store(kv: torch.Tensor, weight: torch.Tensor, eps: float, position
         _need(qp, "qp", cache.dtype, (T, H, D), dev)
     _check(lib.qe_latent_kv_store(kv.data_ptr(), weight.data_ptr(), float(eps), positions.data_ptr(),
                                   inv_freq.data_ptr(), 2 * inv_freq.shape[0], _ptr(slots), cache.data_ptr(),
-                                  _DT[cache.dtype], T, R, D - R, _ptr(q), _ptr(qp), H, int(dim), _stream()), "latent_kv_store")
+                                  _DT[cache.dtype], T, R, D - R, _ptr(q), _ptr(qp), H, int(dim), int(bool(half_split)),
+                                  _stream()), "latent_kv_store")
 
 
 def latent_q_rotate(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, qp: torch.Tensor,
-                    dim: int) -> None:
+                    dim: int, half_split: bool = False) -> None:
     """q [T, H, dim + Dr] -> the last Dr of each head, turned as in latent_kv_store, into the last Dr of
     qp [T, H, R + Dr]."""
     lib = load_library()
@@ -986,16 +992,21 @@ def latent_q_rotate(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Te
     R = qp.shape[2] - Dr
     if Dr < 0 or R <= 0:
         raise KernelError("latent_q_rotate: sizes do not fit")
+    if Dr == 0:
+        return
     _need(positions, "positions", torch.int32, (T,), q.device)
     _need(inv_freq, "inv_freq", torch.float32, (None,), q.device)
     _check(lib.qe_latent_q_rotate(q.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(), 2 * inv_freq.shape[0],
-                                  qp.data_ptr(), _DT[q.dtype], T, H, int(dim), Dr, R, _stream()), "latent_q_rotate")
+                                  qp.data_ptr(), _DT[q.dtype], T, H, int(dim), Dr, R, int(bool(half_split)), _stream()),
+           "latent_q_rotate")
 
 
 def latent_attention(qp: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
-                     block_table: torch.Tensor, latent: int, scale: float, algo: int = ALGO_AUTO) -> torch.Tensor:
+                     block_table: torch.Tensor, latent: int, scale: float, algo: int = ALGO_AUTO,
+                     window: int = 0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """qp [T, H, R + Dr], cache [pages, 1, 1, P, R + Dr]: per (token, head) softmax(scale * qp . rows) . rows[:R]
-    over the rows at positions 0 .. p of request tok_seq[t] -> [T, H, R].  32-bit scores and weights.  The rows
+    over the rows at positions 0 .. p of request tok_seq[t] (``window`` > 0: at p - window + 1 .. p) -> [T, H, R].
+    ``sink`` (float32 [H]): exp(sink[h]) joins the softmax's denominator, one more entry that carries no value.  32-bit scores and weights.  The rows
     of a request are consecutive and their positions rise.  bfloat16 goes to the kernel on the matrix units
     where it takes the sizes (multiples of 8, a latent of at most 512; the weights are rounded to bfloat16
     before they meet the values), everything else (and ALGO_GENERIC) to the kernel on the vector units."""
@@ -1009,17 +1020,23 @@ def latent_attention(qp: torch.Tensor, cache: torch.Tensor, positions: torch.Ten
     _need(positions, "positions", torch.int32, (T,), dev)
     _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
     _need(block_table, "block_table", torch.int32, (None, None), dev)
+    window = int(window or 0)
+    if window < 0:
+        raise KernelError("latent_attention: a negative window")
+    if sink is not None:
+        _need(sink, "sink", torch.float32, (H,), dev)
     out = torch.empty((T, H, R), dtype=qp.dtype, device=dev)
     if qp.dtype == torch.bfloat16 and algo != ALGO_GENERIC and lib.qe_latent_attention_mfma_supported(R, D - R):
-        nbytes = lib.qe_latent_attention_mfma_workspace_bytes(T, H, R)
+        nbytes = lib.qe_latent_attention_mfma_workspace_bytes(T, H, R, window)
         ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev) if nbytes else None
         _check(lib.qe_latent_attention_mfma(qp.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
                                             tok_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, H, R,
-                                            D - R, P, float(scale), _ptr(ws), nbytes, _stream()), "latent_attention (mfma)")
+                                            D - R, P, float(scale), window, _ptr(sink), _ptr(ws), nbytes, _stream()),
+               "latent_attention (mfma)")
         return out
     _check(lib.qe_latent_attention(qp.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
                                    tok_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, H, R, D - R, P,
-                                   float(scale), _DT[qp.dtype], _stream()), "latent_attention")
+                                   float(scale), window, _ptr(sink), _DT[qp.dtype], _stream()), "latent_attention")
     return out
 
 
@@ -1027,7 +1044,7 @@ def gemm_heads(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Option
                algo: int = ALGO_AUTO) -> torch.Tensor:
     """out[t, h, :N] = w[h] x[t, h, :K] for w [H, N, K]; x [T, H, >= K] and out [T, H, >= N] (the product reads
     the first K and writes the first N numbers of each head).  gate [T, H * N]: the result times
-    sigmoid(gate)."""
+    sigmoid(gate); gate [T, H] (or a view of H columns of wider rows): one gate per head."""
     lib = load_library()
     _need(w, "w", _ACT, (None, None, None))
     H, N, K = w.shape
@@ -1038,15 +1055,23 @@ def gemm_heads(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Option
         raise KernelError("gemm_heads: heads narrower than the product")
     if x.dtype == torch.float32 and w.dtype != torch.float32:
         raise KernelError("gemm_heads: 32-bit activations need 32-bit weights")
+    gs = (0, 0, 0)
     if gate is not None:
-        _need(gate, "gate", x.dtype, (T, H * N), x.device)
+        if gate.dim() == 2 and gate.shape == (T, H) and gate.stride(1) == 1 and H * N != H:
+            if not gate.is_cuda or gate.dtype != x.dtype or gate.device != x.device:
+                raise KernelError("gemm_heads: the gate is not where and what the rows are")
+            gs = (gate.stride(0), 1, 0)
+        else:
+            _need(gate, "gate", x.dtype, (T, H * N), x.device)
+            gs = (H * N, N, 1)
     if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and algo != ALGO_GENERIC and
             lib.qe_gemm_heads_mfma_supported(K, H * x.shape[2], x.shape[2])):
         _check(lib.qe_gemm_heads_mfma(x.data_ptr(), H * x.shape[2], x.shape[2], w.data_ptr(), out.data_ptr(),
-                                      H * out.shape[2], out.shape[2], _ptr(gate), T, H, N, K, _stream()), "gemm_heads (mfma)")
+                                      H * out.shape[2], out.shape[2], _ptr(gate), gs[0], gs[1], gs[2], T, H, N, K, _stream()),
+               "gemm_heads (mfma)")
         return out
     _check(lib.qe_gemm_heads(x.data_ptr(), H * x.shape[2], x.shape[2], w.data_ptr(), out.data_ptr(),
-                             H * out.shape[2], out.shape[2], _ptr(gate), T, H, N, K, _DT[x.dtype], _DT[w.dtype],
+                             H * out.shape[2], out.shape[2], _ptr(gate), gs[0], gs[1], gs[2], T, H, N, K, _DT[x.dtype], _DT[w.dtype],
                              _stream()), "gemm_heads")
     return out
 
@@ -1066,18 +1091,29 @@ def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int):
     return ids, weights
 
 
-def moe_route_biased(logits: torch.Tensor, correction: torch.Tensor, top: int, scale: float, transposed: bool = False):
+def moe_route_biased(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, scale: float,
+                     transposed: bool = False, logit_bias: Optional[torch.Tensor] = None, experts: int = 0):
     """logits float32 [T, E] (``transposed``: [E, T]), correction float32 [E] -> (ids int32 [T, top], weights float32 [T, top]): softmax
     over all experts; the ``top`` largest of score + correction are chosen (the lower index on ties); their
-    weights are their scores without the correction, divided by the chosen scores' sum (+ 1e-20), times scale."""
+    weights are their scores without the correction, divided by the chosen scores' sum (+ 1e-20), times scale.
+    Without a correction (None) the ``top`` largest logits are chosen and weighed by the softmax over them alone.
+    ``logit_bias`` (float32 [E]) is added to the logits first.  ``experts``: only the first so many outputs of the
+    logits are the router's (the rest belongs to the caller); 0: all."""
     lib = load_library()
     _need(logits, "logits", torch.float32, (None, None))
-    T, E = (logits.shape[1], logits.shape[0]) if transposed else logits.shape
-    _need(correction, "correction", torch.float32, (E,), logits.device)
+    T, ld = (logits.shape[1], 0) if transposed else logits.shape
+    E = int(experts) or (logits.shape[0] if transposed else logits.shape[1])
+    if E > (logits.shape[0] if transposed else logits.shape[1]):
+        raise KernelError("moe_route_biased: more experts than logits")
+    if correction is not None:
+        _need(correction, "correction", torch.float32, (E,), logits.device)
+    if logit_bias is not None:
+        _need(logit_bias, "logit_bias", torch.float32, (E,), logits.device)
     ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
-    _check(lib.qe_moe_route_biased(logits.data_ptr(), correction.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E,
-                                   int(top), float(scale), int(bool(transposed)), _stream()), "moe_route_biased")
+    _check(lib.qe_moe_route_biased(logits.data_ptr(), _ptr(correction), ids.data_ptr(), weights.data_ptr(), T, E,
+                                   int(top), float(scale), int(bool(transposed)), _ptr(logit_bias), int(ld), _stream()),
+           "moe_route_biased")
     return ids, weights
 
 
@@ -1149,8 +1185,10 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
     weighed and added in 32-bit (float32, or bfloat16 with bfloat16 operands: half the bytes of the largest tensor of
     the mixture).  ``biased_route``: instead of ids and weights (both None), (logits float32 [T, E + identity],
     correction float32 [E + identity], top, scale[, transposed: the logits are [E + identity, T]]) for the routing of
-    moe_route_biased: a step of few tokens then
-    routes, sorts and writes the identity experts' rows in one launch.  ``parts_out``: float32 [top, T, H] to take the
+    moe_route_biased (a None correction: the largest logits, weighed by the softmax over them alone; two more entries:
+    a bias float32 [E + identity] that is added to the logits, and how many of the logits' outputs are the router's
+    where they are the first of more): a step of few tokens then
+    routes, sorts and writes the identity experts' rows in one launch.  ``limit`` 0: the plain silu(g) u.  ``parts_out``: float32 [top, T, H] to take the
     parts (the paths of fewer than 1024 pairs only).
 
     The (token, choice) pairs are grouped by expert on the device.  bfloat16 with many pairs: their rows are
@@ -1167,10 +1205,18 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
             raise KernelError("moe_experts: ids and weights, or a route to compute them, not both")
         r_logits, r_corr, top, r_scale = biased_route[:4]
         r_transposed = len(biased_route) > 4 and bool(biased_route[4])       # logits [E + identity, T]
+        r_bias = biased_route[5] if len(biased_route) > 5 else None          # added to the logits (float32, an entry per output)
         top = int(top)
         _need(r_logits, "logits", torch.float32, (None, T) if r_transposed else (T, None), dev)
-        r_outputs = r_logits.shape[0] if r_transposed else r_logits.shape[1]
-        _need(r_corr, "correction", torch.float32, (r_outputs,), dev)
+        r_width = r_logits.shape[0] if r_transposed else r_logits.shape[1]
+        # (the router's outputs may be the first of more outputs of one product)
+        r_outputs = int(biased_route[6]) if len(biased_route) > 6 and biased_route[6] else r_width
+        if r_outputs > r_width:
+            raise KernelError("moe_experts: more router outputs than logits")
+        if r_corr is not None:
+            _need(r_corr, "correction", torch.float32, (r_outputs,), dev)
+        if r_bias is not None:
+            _need(r_bias, "logit_bias", torch.float32, (r_outputs,), dev)
     else:
         _need(ids, "ids", torch.int32, (T, None), dev)
         top = ids.shape[1]
@@ -1218,13 +1264,15 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
             weights = torch.empty((T, top), dtype=torch.float32, device=dev)
             if parts is None:
                 parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
-            _check(lib.qe_moe_front_small(r_logits.data_ptr(), r_corr.data_ptr(), x.data_ptr(), ids.data_ptr(),
+            _check(lib.qe_moe_front_small(r_logits.data_ptr(), _ptr(r_corr), x.data_ptr(), ids.data_ptr(),
                                           weights.data_ptr(), perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
                                           n_tiles.data_ptr(), parts.data_ptr(), max_tiles, T, Hout, E + identity, E, top,
-                                          float(r_scale), tile_rows, _DT[x.dtype], _stream()), "moe_front_small")
+                                          float(r_scale), tile_rows, _DT[x.dtype], _ptr(r_bias), r_width, _stream()),
+                   "moe_front_small")
             fused_front = True
         else:
-            ids, weights = moe_route_biased(r_logits, r_corr, top, r_scale, transposed=r_transposed)
+            ids, weights = moe_route_biased(r_logits, r_corr, top, r_scale, transposed=r_transposed, logit_bias=r_bias,
+                                            experts=r_outputs)
     # (identity experts are buckets of the sort like the others, behind them, and get no tiles)
     if not fused_front:
         _check(lib.qe_moe_sort(ids.data_ptr(), n, E + identity, E, tile_rows, perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
@@ -1298,7 +1346,7 @@ def qkv_norm_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, k_dim: 
     T, dev = qkv.shape[0], qkv.device
     Hq, Hkv, Dk, Dv = int(num_heads), int(num_kv_heads), int(k_dim), int(v_dim)
     need = Hq * Dk + Hkv * Dk + (0 if values_from_keys else Hkv * Dv)
-    if qkv.shape[1] != need:
+    if qkv.shape[1] < need:          # (rows may go on behind q | k | v: other outputs of the same product)
         raise KernelError(f"qkv_norm_store: rows of {qkv.shape[1]} numbers, {need} expected")
     _need(cache, "cache", qkv.dtype, (None, 2, Hkv, None, None), dev)
     P, Dc = cache.shape[3], cache.shape[4]
@@ -1524,3 +1572,36 @@ def scaled_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float) -> torch.
     _check(lib.qe_scaled_sum(a.data_ptr(), float(sa), b.data_ptr(), float(sb), _DT[a.dtype], y.data_ptr(), a.numel(),
                              _stream()), "scaled_sum")
     return y
+
+
+def moe_row_gate(dst: torch.Tensor, src: torch.Tensor, gate_logits: torch.Tensor, accumulate: bool) -> None:
+    """dst[t] (+)= sigmoid(gate_logits[t]) * src[t]: dst float32 [T, H], src [T, H] (may be dst itself), gate_logits
+    float32 [T] or a column of wider rows.  An expert that every token uses, weighed by one number a token."""
+    lib = load_library()
+    _need(dst, "dst", torch.float32, (None, None))
+    T, H = dst.shape
+    _need(src, "src", _ACT, (T, H), dst.device)
+    if gate_logits.dtype != torch.float32 or gate_logits.dim() != 1 or gate_logits.shape[0] != T or not gate_logits.is_cuda:
+        raise KernelError("moe_row_gate: one 32-bit gate a row")
+    _check(lib.qe_moe_row_gate(dst.data_ptr(), src.data_ptr(), _DT[src.dtype], gate_logits.data_ptr(),
+                               max(1, gate_logits.stride(0)), T, H, int(bool(accumulate)), _stream()), "moe_row_gate")
+
+
+def diff_heads(a: torch.Tensor, num_heads: int, num_kv_heads: int, v_dim: int, lam: float, eps: float, out_scale: float,
+               gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Joins the two maps of differential attention: a [T, 2 H, Dc], map m of head h = g (H / G) + j at query head
+    g (2 H / G) + m (H / G) + j -> out [T, H, v_dim]: o = a1 - lam a2, divided by its root mean square over v_dim
+    (eps inside the root), times out_scale, times sigmoid(gate[t, h]) (gate [T, H], or H columns of wider rows)."""
+    lib = load_library()
+    _need(a, "a", _ACT, (None, 2 * int(num_heads), None))
+    T, _, Dc = a.shape
+    H, G, Dv = int(num_heads), int(num_kv_heads), int(v_dim)
+    gs = 0
+    if gate is not None:
+        if gate.dim() != 2 or gate.shape != (T, H) or gate.stride(1) != 1 or gate.dtype != a.dtype or gate.device != a.device:
+            raise KernelError("diff_heads: one gate a head, in the rows' element type")
+        gs = gate.stride(0)
+    out = torch.empty((T, H, Dv), dtype=a.dtype, device=a.device)
+    _check(lib.qe_diff_heads(a.data_ptr(), out.data_ptr(), _ptr(gate), gs, T, H, G, Dv, Dc, float(lam), float(eps),
+                             float(out_scale), _DT[a.dtype], _stream()), "diff_heads")
+    return out

@@ -1,4 +1,4 @@
 from .base import CacheBinding, Runtime, TensorInfo
 from .registry import build_part, part_class, register_part, unregister_part
-from . import norm, rope, attention, mlp, block, conv, latent_attention, moe, recurrent  # registers the built-in parts
+from . import norm, rope, attention, mlp, block, conv, latent_attention, moe, recurrent, diff_attention  # registers the built-in parts
 from .model import DecoderModel, cache_plan, expected_tensors

@@ -23,13 +23,14 @@ class PreNormBlock:
         self.hidden = int(hidden_size)
         self.mixer_norm = build_part(spec.mixer_norm, hidden_size)
         self.mixer = build_part(spec.mixer, hidden_size)
-        self.ffn_norm = build_part(spec.ffn_norm, hidden_size)
-        self.ffn = build_part(spec.ffn, hidden_size)
+        # (a layer without a feed-forward is its mixer alone; its second norm then has nothing to stand before)
+        self.ffn = build_part(spec.ffn, hidden_size) if spec.ffn is not None else None
+        self.ffn_norm = build_part(spec.ffn_norm, hidden_size) if self.ffn is not None else None
 
     @property
     def graph_safe(self) -> bool:
         """False if any part of the block says that its forward cannot be recorded into a graph."""
-        return all(getattr(p, "graph_safe", True) for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn))
+        return all(getattr(p, "graph_safe", True) for p in self.parts())
 
     @property
     def graph_safe_with_state(self) -> bool:
@@ -37,7 +38,15 @@ class PreNormBlock:
         return getattr(self.mixer, "graph_safe", False) is True
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None)
+
+    @staticmethod
+    def _named(spec):
+        """(checkpoint name, part spec) of the block's parts."""
+        out = [(_names(spec)[0], spec.mixer_norm), (_names(spec)[1], spec.mixer)]
+        if spec.ffn is not None:
+            out += [(_names(spec)[2], spec.ffn_norm), (_names(spec)[3], spec.ffn)]
+        return out
 
     @staticmethod
     def cache_needs(spec, hidden: int):
@@ -51,14 +60,18 @@ class PreNormBlock:
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
         out: Dict[str, TensorInfo] = {}
-        for name, sub in zip(_names(spec), (spec.mixer_norm, spec.mixer, spec.ffn_norm, spec.ffn)):
+        for name, sub in PreNormBlock._named(spec):
             for rel, info in part_class(sub.kind).expected_tensors(sub, hidden).items():
-                out[f"{name}.{rel}"] = info
+                out[join_name(name, rel)] = info
         return out
 
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
-        for name, part in zip(_names(self.spec), (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)):
-            part.load(sub_tensors(tensors, name + "."), rt)
+        for (name, sub), part in zip(self._named(self.spec), self.parts()):
+            names = type(part).expected_tensors(sub, self.hidden)
+            if "" in names:        # (a part that is one tensor, which carries the part's own name)
+                part.load(named_tensors(tensors, name, names), rt)
+            else:
+                part.load(sub_tensors(tensors, name + "."), rt)
 
     def forward(self, h, pending: Optional[torch.Tensor], ctx, bindings) -> torch.Tensor:
         """h: the 32-bit residual stream, a tensor (updated in place) or a Stream (whose buffers may
@@ -69,6 +82,8 @@ class PreNormBlock:
         stream = h if isinstance(h, Stream) else Stream(h)
         x = self._input(self.mixer_norm, self.mixer, stream, pending, ctx)
         a = self.mixer.forward(x, ctx, bindings[0])
+        if self.ffn is None:
+            return a
         x = self._input(self.ffn_norm, self.ffn, stream, a, ctx)
         return self.ffn.forward(x, ctx)
 

@@ -19,27 +19,38 @@ class SwiGLU:
     def __init__(self, spec, hidden_size: int):
         self.hidden = int(hidden_size)
         self.inter = int(spec.intermediate_size)
+        self.names = tuple(spec.names)
         self.w_gu = self.w_down = None
         self.interleaved = False
 
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
         i = spec.intermediate_size
+        gate, up, down = spec.names
         return {
-            "gate_proj.weight": TensorInfo((i, hidden)),
-            "up_proj.weight": TensorInfo((i, hidden)),
-            "down_proj.weight": TensorInfo((hidden, i)),
+            gate: TensorInfo((i, hidden)),
+            up: TensorInfo((i, hidden)),
+            down: TensorInfo((hidden, i)),
         }
 
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        n_gate, n_up, n_down = self.names
+        g, u = tensors[n_gate], tensors[n_up]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
         # gate and up rows in alternating blocks of 32, so that a product's epilogue finds the gate
         # and the up of an output side by side; widths that are no multiple of 32 keep gate | up
         self.interleaved = self.inter % 32 == 0
         self.w_gu = rt.place_matrix(ops.interleave_gate_up(g, u) if self.interleaved else torch.cat([g, u], dim=0))
-        self.w_down = rt.place_matrix(tensors["down_proj.weight"])
+        self.w_down = rt.place_matrix(tensors[n_down])
+
+    def activation(self, x) -> torch.Tensor:
+        """silu(gate x) * up x [T, I] in the activation type, for x [T, H] (not a StreamInput)."""
+        if self.interleaved and ops.gemm_silu_supported(x, self.w_gu):
+            return ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL_IL)
+        if not self.interleaved and ops.gemm_fused_supported(x, self.w_gu):
+            return ops.gemm(x, self.w_gu, epilogue=ops.EPI_SILU_MUL)
+        return ops.silu_mul(ops.gemm(x, self.w_gu), interleaved=self.interleaved)
 
     def forward(self, x, ctx) -> torch.Tensor:
         """Returns the feed-forward output [T, H], or float32 partial products [S, T, H] of it.

@@ -77,6 +77,28 @@ class BareRMSNorm(RMSNorm):
         self.weight = rt.place_vector(tensors[""])
 
 
+class BareLayerNorm:
+    """Layer norm with a weight and no bias, (v - mean) * rsqrt(mean of the squared deviations + eps) * w, the weight
+    tensor named as the part itself.  The residual sum that stands before it is formed in the same kernel, as in the
+    RMS norms; it is no product's prologue (no ``fusable_weight``)."""
+
+    def __init__(self, spec, size: int):
+        self.eps = float(spec.eps)
+        self.size = int(size)
+        self.weight: Optional[torch.Tensor] = None
+
+    @staticmethod
+    def expected_tensors(spec, size: int) -> Dict[str, TensorInfo]:
+        return {"": TensorInfo((size,), "ones", "vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.weight = rt.place_vector(tensors[""])
+
+    def forward(self, h: torch.Tensor, rt: Runtime, delta: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.rmsnorm(h, self.weight, self.eps, rt.dtype, delta=delta, rows=rows, center=True)
+
+
 class StreamScale:
     """Multiplies the 32-bit stream right after the embedding by one number."""
 
@@ -116,5 +138,6 @@ class LogitSoftcap:
 register_part("rmsnorm", RMSNorm)
 register_part("logit_softcap", LogitSoftcap)
 register_part("rmsnorm_bare", BareRMSNorm)
+register_part("layernorm_bare", BareLayerNorm)
 register_part("stream_scale", StreamScale)
 register_part("rmsnorm_scalar", ScalarRMSNorm)

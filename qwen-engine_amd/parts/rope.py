@@ -65,13 +65,17 @@ class RotaryPairs:
 class RotaryHalfAngles:
     """Half-split rotation of a head's first ``rotary_dim`` numbers (number i pairs with i + rotary_dim / 2) by
     position * theta^(-2i / rotary_dim).  The kernels that rotate form the angle, its sine and cosine in 32-bit from
-    ``inv_freq()``; the frequencies are computed in 64-bit and rounded once.  No table: no limit of positions."""
+    ``inv_freq()``; the frequencies are computed in 64-bit, divided by the spec's scaling factor and rounded once.
+    No table: no limit of positions."""
 
     def __init__(self, spec, hidden_size: int = 0):
         self.theta = float(spec.theta)
         self.rotary_dim = int(spec.rotary_dim)
         if self.rotary_dim % 2 or self.rotary_dim <= 0:
             raise ValueError(f"rotary_dim {self.rotary_dim} is odd or not positive")
+        self.scaling_factor = float(getattr(spec, "scaling_factor", 1.0))
+        if not self.scaling_factor > 0:
+            raise ValueError(f"a scaling factor of {self.scaling_factor}")
         self._inv_freq: Optional[torch.Tensor] = None
 
     @staticmethod
@@ -81,7 +85,8 @@ class RotaryHalfAngles:
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
         d = self.rotary_dim
         i = torch.arange(0, d, 2, dtype=torch.float64)
-        self._inv_freq = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -i / d).to(torch.float32).to(rt.device)
+        f = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -i / d) / self.scaling_factor
+        self._inv_freq = f.to(torch.float32).to(rt.device)
 
     def inv_freq(self) -> torch.Tensor:
         return self._inv_freq
