@@ -35,8 +35,9 @@ Other sizes and workloads (not what the default line reports):
                             recorded graph of repetitions over weights that do not fit the caches, and its rate
                             against the nominal and the measured peaks (the counterpart of the reference's
                             per-operator benchmarks, src/layers/ops/linear.py:204-249)
-  --design zarorax|nufavik|potatar
-                            another design beside the closest Qwen3 model of equal sizes (width, layers, heads, and a
+  --design zarorax|nufavik|potatar|safurax
+                            another design beside the closest Qwen3 model of equal sizes (safurax: beside the Zarorax
+                            model of equal sizes, the engine's other design of latent attention and routed experts) (width, layers, heads, and a
                             feed-forward as wide as the experts a token uses, or of as many weights): prefill (one prompt of --prefill-tokens
                             in one step) and decode (batch 1 and --batch at --context) of both, at the sizes of
                             --design-sizes (small, medium); one JSON line of its own.  The default line is unchanged.
@@ -95,7 +96,7 @@ def parse():
                     help="run steps of single new tokens beside a prompt portion as they come, not from a recorded graph")
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
     ap.add_argument("--kernels", action="store_true", help="time each kernel of a layer alone over a range of rows")
-    ap.add_argument("--design", default=None, choices=["zarorax", "nufavik", "potatar"],
+    ap.add_argument("--design", default=None, choices=["zarorax", "nufavik", "potatar", "safurax"],
                     help="measure this design beside the closest Qwen3 model of equal sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes (small, medium), with commas")
     ap.add_argument("--warmup-passes", type=int, default=2,
@@ -418,6 +419,40 @@ def potatar_config(z, layers, vocab):
             "norm": {"eps": 1e-5}, "layers": [order[i % 4] for i in range(layers)]}
 
 
+# Layer sizes for --design safurax: those of --design zarorax (latent attention, experts), a window for the layers with
+# direct queries, key/value heads and the size of a map for the differential layers, the shared expert's width
+SAFURAX_SIZES = {
+    "small": dict(ZARORAX_SIZES["small"], window=1024, kv_heads=4, map_dim=64, shared_ff=768),
+    "medium": dict(ZARORAX_SIZES["medium"], window=1024, kv_heads=4, map_dim=128, shared_ff=1024),
+}
+
+
+def safurax_config(z, layers, vocab):
+    """A dense layer first, then mixtures; the mixers in turn: a query latent, direct queries under a window, the same on
+    that layer's latent, differential attention."""
+    la1 = {"heads": z["heads"], "dim": z["dim"], "vdim": z["vdim"], "kv_rank": z["kv_rank"], "q_rank": z["q_rank"],
+           "scale": z["dim"] ** -0.5}
+    la2 = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["vdim"], "kv_rank": z["kv_rank"],
+           "scale": (z["dim"] + z["rot_dim"]) ** -0.5, "rot": {"base": 10000.0, "dims": z["rot_dim"]},
+           "mask": {"size": z["window"]}}
+    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["map_dim"], "vdim": z["vdim"], "diff": 0.5,
+           "scale": z["map_dim"] ** -0.5, "rot": {"base": 10000.0, "dims": z["map_dim"] // 2, "scaling": {"factor": 4.0}}}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "router": {"experts": z["experts"], "top": z["top"]},
+           "shared": {"ff": z["shared_ff"]}}
+    ls = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            layer = {"type": "latent_attention", "mixer": la1}
+        elif kind == 3:
+            layer = {"type": "attention", "mixer": att}
+        else:
+            layer = {"type": "latent_attention_2", "mixer": dict(la2, kv_from=i - 1) if kind == 2 else la2}
+        ls.append(dict(layer, mlp={"kind": "dense", "ff": z["ff"]} if i == 0 else moe))
+    return {"architecture": "Safurax", "vocab": vocab, "width": z["width"], "embedding": {"scale": 4.0}, "norm": {"eps": 1e-5},
+            "layers": ls}
+
+
 def design_compare(args) -> int:
     """Prefill and decode of another design beside the Qwen3 model of equal sizes, through the same step
     function.  A "step" is one decode step; the line's value is the design's decode rate at --batch, first size."""
@@ -485,7 +520,14 @@ def design_compare(args) -> int:
     out = {}
     design = args.design
     title = design.capitalize()
+    other, other_title = ("zarorax", "Zarorax") if design == "safurax" else ("qwen3", "Qwen3")
     for name in [n for n in args.design_sizes.split(",") if n]:
+        if design == "safurax":
+            z = SAFURAX_SIZES[name]
+            out[name] = {"sizes": dict(z, layers=layers, vocab=V), design: measure(config_from_dict(safurax_config(z, layers, V))),
+                         other: measure(config_from_dict(zarorax_config(z, layers, V)))}
+            print(f"[bench] {name}: {out[name]}", file=sys.stderr, flush=True)
+            continue
         if design == "potatar":
             z = POTATAR_SIZES[name]
             zcfg = config_from_dict(potatar_config(z, layers, V))
@@ -505,12 +547,12 @@ def design_compare(args) -> int:
         out[name] = {"sizes": dict(z, layers=layers, vocab=V), design: measure(zcfg), "qwen3": measure(qcfg)}
         print(f"[bench] {name}: {out[name]}", file=sys.stderr, flush=True)
     first = next(iter(out.values()))
-    line = {"metric": f"decode tok/s @ batch {args.batch} ({title}, context {args.context}) beside Qwen3 of equal sizes",
+    line = {"metric": f"decode tok/s @ batch {args.batch} ({title}, context {args.context}) beside {other_title} of equal sizes",
             "value": first[design][f"decode_b{args.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": first[design][f"decode_b{args.batch}_ms_per_step"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
             "data": "synthetic: random weights, uniform-random token ids",
-            "config": {"model": f"{title} and Qwen3 layer sizes (random weights)", "global_batch": args.batch,
+            "config": {"model": f"{title} and {other_title} layer sizes (random weights)", "global_batch": args.batch,
                        "seq_len": args.context, "prefill_tokens": args.prefill_tokens, "page_size": P, "parallelism": "single GPU"},
             "designs": out}
     print(json.dumps(line), flush=True)
