@@ -69,7 +69,29 @@ SC = {
          "mlp": {"kind": "dense", "ff": 40}},
     ],
 }
-TINY = {"A": (SA, 21, 8), "B": (SB, 22, 16), "C": (SC, 23, 4)}      # config, seed, page size
+# D: sizes that fill no tile of any kernel: a width of 72, a latent of 20 with 6 rotated numbers, maps of 12 numbers,
+# three heads on three key/value heads, a differential layer first, a reader two layers behind the latent it reads.
+SD = {
+    "architecture": "Safurax", "vocab": 97, "width": 72, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-4},
+    "layers": [
+        {"type": "attention",
+         "mixer": {"heads": 6, "kv_heads": 3, "dim": 12, "vdim": 20, "diff": 0.6, "scale": 0.29,
+                   "rot": {"base": 300.0, "dims": 4, "scaling": {"factor": 1.5}}},
+         "mlp": {"kind": "dense", "ff": 52}},
+        {"type": "latent_attention_2",
+         "mixer": {"heads": 3, "dim": 10, "rot_dim": 6, "vdim": 12, "kv_rank": 20, "scale": 0.25,
+                   "rot": {"base": 2000.0, "dims": 6}, "mask": {"size": 21}},
+         "mlp": {"kind": "moe", "expert": {"ff": 20}, "router": {"experts": 7, "top": 2}, "shared": {"ff": 12}}},
+        {"type": "latent_attention",
+         "mixer": {"heads": 2, "dim": 18, "vdim": 10, "kv_rank": 28, "q_rank": 12, "scale": 0.2},
+         "mlp": {"kind": "dense", "ff": 36}},
+        {"type": "latent_attention_2",
+         "mixer": {"heads": 5, "dim": 4, "rot_dim": 6, "vdim": 6, "kv_rank": 20, "scale": 0.3, "kv_from": 1,
+                   "rot": {"base": 2000.0, "dims": 6}, "mask": {"size": 21}},
+         "mlp": {"kind": "dense", "ff": 44}},
+    ],
+}
+TINY = {"A": (SA, 21, 8), "B": (SB, 22, 16), "C": (SC, 23, 4), "D": (SD, 24, 2)}      # config, seed, page size
 
 
 def tensor_shapes(cfg):
