@@ -10,8 +10,10 @@
 //   * q written with heads of Dc numbers (zeros beyond a head's own), k and v written into the cache page of
 //     the token's slot, value tiles transposed ([Dc][P], what the engine's attention kernels read) or as rows
 //     ([P][Dc]).
-// One block per token; the row passes through shared memory in 32-bit, all arithmetic in 32-bit, one rounding
-// at the stores.
+// One block per token, or, where heads are normed by themselves and the rows are few, one block per token and group of
+// heads (gridDim.y groups: a group's query heads, its key heads and its value heads; a single row's time is the length
+// of the walk through it, not its bytes); the row passes through shared memory in 32-bit, all arithmetic in 32-bit,
+// one rounding at the stores.
 #include "common.h"
 
 enum { QKN_NONE = 0, QKN_HEAD = 1, QKN_WHOLE = 2 };
@@ -23,19 +25,23 @@ __global__ __launch_bounds__(256) void qkv_norm_store_kernel(
     const float* __restrict__ v_blend, float* __restrict__ v_first, int v_first_write,
     const int* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dims,
     const int* __restrict__ slots, TA* __restrict__ q_out, TA* __restrict__ cache,
-    int Hq, int Hkv, int Dk, int Dv, int Dc, int P, int v_rows) {
+    int HqT, int HkvT, int Dk, int Dv, int Dc, int P, int v_rows) {
     extern __shared__ float sm[];
     __shared__ float red[16];
     const long t = blockIdx.x;
+    // this block's heads: all of them, or one of gridDim.y equal groups
+    const int Hq = HqT / (int)gridDim.y, Hkv = HkvT / (int)gridDim.y;
+    const int q0 = (int)blockIdx.y * Hq, k0 = (int)blockIdx.y * Hkv;
     const int Nq = Hq * Dk, Nk = Hkv * Dk, Nv = Hkv * Dv;
     float* sq = sm;              // Nq
     float* sk = sm + Nq;         // Nk
     float* sv = sk + Nk;         // Nv
     const TA* row = qkv + t * row_stride;
     const int tid = threadIdx.x, nt = blockDim.x;
-    for (int c = tid; c < Nq + Nk; c += nt) sm[c] = Elem<TA>::load(row + c);
+    for (int c = tid; c < Nq; c += nt) sq[c] = Elem<TA>::load(row + q0 * Dk + c);
+    for (int c = tid; c < Nk; c += nt) sk[c] = Elem<TA>::load(row + HqT * Dk + k0 * Dk + c);
     if (!values_from_keys)
-        for (int c = tid; c < Nv; c += nt) sv[c] = Elem<TA>::load(row + Nq + Nk + c);
+        for (int c = tid; c < Nv; c += nt) sv[c] = Elem<TA>::load(row + (HqT + HkvT) * Dk + k0 * Dv + c);
     __syncthreads();
     if (values_from_keys) {      // the keys as projected (Dv == Dk)
         for (int c = tid; c < Nv; c += nt) sv[c] = sk[c];
@@ -79,7 +85,7 @@ __global__ __launch_bounds__(256) void qkv_norm_store_kernel(
         __syncthreads();
     }
     if (v_first) {
-        float* vf = v_first + t * Nv;
+        float* vf = v_first + t * ((long)HkvT * Dv) + k0 * Dv;
         if (v_first_write) {
             for (int c = tid; c < Nv; c += nt) vf[c] = sv[c];
         } else {
@@ -102,7 +108,7 @@ __global__ __launch_bounds__(256) void qkv_norm_store_kernel(
         __syncthreads();
     }
     // ---- stores -------------------------------------------------------------------------------
-    TA* qo = q_out + t * (long)Hq * Dc;
+    TA* qo = q_out + (t * (long)HqT + q0) * Dc;
     for (int i = tid; i < Hq * Dc; i += nt) {
         const int h = i / Dc, d = i - h * Dc;
         Elem<TA>::store(qo + i, d < Dk ? sq[h * Dk + d] : 0.f);
@@ -111,14 +117,15 @@ __global__ __launch_bounds__(256) void qkv_norm_store_kernel(
     if (slot < 0) return;                                  // (a row that writes nowhere)
     const long page = slot / P;
     const int off = slot % P;
-    TA* kp = cache + page * (2L * Hkv * P * Dc);
-    TA* vp = kp + (long)Hkv * P * Dc;
+    TA* kp = cache + page * (2L * HkvT * P * Dc);
+    TA* vp = kp + (long)HkvT * P * Dc;
     for (int i = tid; i < Hkv * Dc; i += nt) {
         const int h = i / Dc, d = i - h * Dc;
-        Elem<TA>::store(kp + ((long)h * P + off) * Dc + d, d < Dk ? sk[h * Dk + d] : 0.f);
+        const long hc = h + k0;                                // the head's place among all key/value heads
+        Elem<TA>::store(kp + (hc * P + off) * Dc + d, d < Dk ? sk[h * Dk + d] : 0.f);
         const float v = d < Dv ? sv[h * Dv + d] : 0.f;
-        if (v_rows) Elem<TA>::store(vp + ((long)h * P + off) * Dc + d, v);
-        else Elem<TA>::store(vp + ((long)h * Dc + d) * P + off, v);
+        if (v_rows) Elem<TA>::store(vp + (hc * P + off) * Dc + d, v);
+        else Elem<TA>::store(vp + (hc * Dc + d) * P + off, v);
     }
 }
 
@@ -141,13 +148,17 @@ extern "C" int qe_qkv_norm_store(const void* qkv, int row_stride, const float* q
     const int need = Hq * Dk + Hkv * Dk + (values_from_keys ? 0 : Hkv * Dv);
     QE_REQUIRE(row_stride >= need, "qkv_norm_store: rows of %d numbers, %d needed", row_stride, need);
     if (T == 0) return 0;
-    const size_t shmem = (size_t)(Hq * Dk + Hkv * Dk + Hkv * Dv) * sizeof(float);
+    // Few rows, heads normed by themselves (or not at all): a block per token and key/value head with its query heads
+    int groups = 1;
+    if (qk_mode != QKN_WHOLE && T < 512 && Hkv > 1 && Hq % Hkv == 0) groups = Hkv;
+    const size_t shmem = (size_t)(Hq * Dk + Hkv * Dk + Hkv * Dv) / groups * sizeof(float);
     QE_REQUIRE(shmem <= 150 * 1024, "qkv_norm_store: a row of %zu bytes does not fit shared memory", shmem);
+    const dim3 grid(T, groups);
 #define QE_QNS(TA_)                                                                                                  \
     do {                                                                                                             \
         if (shmem > 48 * 1024)                                                                                       \
             (void)hipFuncSetAttribute((const void*)qkv_norm_store_kernel<TA_>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem); \
-        qkv_norm_store_kernel<TA_><<<T, 256, shmem, stream>>>(                                                       \
+        qkv_norm_store_kernel<TA_><<<grid, 256, shmem, stream>>>(                                                       \
             (const TA_*)qkv, row_stride, q_w, k_w, qk_mode, qk_eps, values_from_keys, v_eps, v_norm, v_blend, v_first, \
             v_first_write, positions, inv_freq, rot_dims, slots, (TA_*)q_out, (TA_*)cache, Hq, Hkv, Dk, Dv, Dc, P,   \
             v_rows);                                                                                                 \
