@@ -435,7 +435,7 @@ def safurax_config(z, layers, vocab):
     la2 = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["vdim"], "kv_rank": z["kv_rank"],
            "scale": (z["dim"] + z["rot_dim"]) ** -0.5, "rot": {"base": 10000.0, "dims": z["rot_dim"]},
            "mask": {"size": z["window"]}}
-    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["map_dim"], "vdim": z["vdim"], "diff": 0.5,
+    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["map_dim"], "vdim": z["vdim"], "diff": 0.4,
            "scale": z["map_dim"] ** -0.5, "rot": {"base": 10000.0, "dims": z["map_dim"] // 2, "scaling": {"factor": 4.0}}}
     moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "router": {"experts": z["experts"], "top": z["top"]},
            "shared": {"ff": z["shared_ff"]}}
