@@ -4,6 +4,7 @@ written as model folders.  Sizes differ from one another wherever the design all
 import json
 import math
 import os
+import random
 
 import torch
 
@@ -92,6 +93,53 @@ SD = {
     ],
 }
 TINY = {"A": (SA, 21, 8), "B": (SB, 22, 16), "C": (SC, 23, 4), "D": (SD, 24, 2)}      # config, seed, page size
+
+
+def random_config(seed):
+    """A Safurax configuration drawn at random: two to seven layers of the three mixers in any order (layers on an
+    earlier layer's latent among them), head counts, sizes, windows, constants and feed-forwards drawn independently."""
+    rng = random.Random(seed)
+    width = rng.choice([64, 80, 96, 128, 160, 192, 256, 320, 384, 512])
+    n_layers = rng.randint(2, 7)
+    layers = []
+    la2_own = []
+    for i in range(n_layers):
+        kind = rng.choice(["latent_attention", "latent_attention_2", "latent_attention_2", "attention"])
+        heads = rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 24])
+        dim = rng.choice([8, 16, 24, 32, 48, 64, 96, 128])
+        vdim = rng.choice([8, 16, 24, 32, 48, 64, 96, 128])
+        if kind == "latent_attention":
+            m = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": rng.choice([16, 24, 32, 64, 96, 128, 192, 256, 320]),
+                 "q_rank": rng.choice([16, 32, 48, 64, 128, 192]), "scale": dim ** -0.5}
+        elif kind == "latent_attention_2":
+            if la2_own and rng.random() < 0.4:
+                j = rng.choice(la2_own)
+                src = layers[j]["mixer"]
+                m = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": src["kv_rank"], "rot_dim": src["rot_dim"],
+                     "rot": dict(src["rot"]), "scale": (dim + src["rot_dim"]) ** -0.5, "mask": {"size": rng.randint(1, 300)}, "kv_from": j}
+            else:
+                rd = rng.choice([2, 4, 8, 16, 32, 64])
+                m = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": rng.choice([16, 24, 32, 64, 96, 128, 192, 256, 320]), "rot_dim": rd,
+                     "rot": {"base": rng.choice([100.0, 10000.0, 50000.0, 1e6]), "dims": rd}, "scale": (dim + rd) ** -0.5,
+                     "mask": {"size": rng.randint(1, 300)}}
+                la2_own.append(i)
+        else:
+            kvh = rng.choice([d for d in (1, 2, 3, 4, 6, 8) if heads % d == 0])
+            dims = rng.choice([d for d in (2, 4, 8, 16, 32, 64, 128) if d <= dim])
+            m = {"heads": heads, "kv_heads": kvh, "dim": dim, "vdim": vdim, "diff": rng.choice([0.1, 0.2, 0.5, 0.8]),
+                 "scale": dim ** -0.5, "rot": {"base": rng.choice([1000.0, 20000.0]), "dims": dims, "scaling": {"factor": rng.choice([1.0, 2.0, 8.0])}}}
+        r = rng.random()
+        if r < 0.45:
+            mlp = {"kind": "dense", "ff": rng.choice([40, 64, 100, 128, 320, 512, 768])}
+        elif r < 0.95:
+            e = rng.choice([2, 3, 4, 8, 16, 32, 64, 96])
+            mlp = {"kind": "moe", "expert": {"ff": rng.choice([16, 24, 32, 64, 96, 128, 160])},
+                   "router": {"experts": e, "top": rng.randint(1, min(e, 8))}, "shared": {"ff": rng.choice([16, 32, 64, 96, 128])}}
+        else:
+            mlp = None
+        layers.append({"type": kind, "mixer": m, "mlp": mlp})
+    return {"architecture": "Safurax", "vocab": rng.choice([128, 300, 512, 1000]), "width": width,
+            "embedding": {"scale": rng.choice([1.0, 4.0, 12.0])}, "norm": {"eps": rng.choice([1e-6, 1e-5, 1e-3])}, "layers": layers}
 
 
 def tensor_shapes(cfg):

@@ -9,7 +9,7 @@ import torch
 import qwen_engine_amd  # noqa: F401
 from plain import safurax_plain as S
 import traces
-from safurax_tiny import SA, TINY, make_folder, random_tensors, write_folder
+from safurax_tiny import SA, TINY, make_folder, random_config, random_tensors, write_folder
 
 pytestmark = pytest.mark.gpu
 
@@ -302,6 +302,22 @@ def test_middling_sizes_on_the_matrix_unit_kernels(tmp_path):
                 assert bad is None, f"{cut}: first wrong logits at (request, position, relative error) {bad}"
             else:
                 _assert_close_but_for_close_calls(got, ref, f"{dtype} {cut}")
+
+
+@pytest.mark.parametrize("seed", [3, 4, 5, 11, 24, 27])
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Layer orders, head counts, sizes, windows and constants that no other test names, in float32 against the plain
+    model, whole and in a mixed schedule."""
+    cfg = random_config(seed)
+    folder = write_folder(str(tmp_path / "model"), cfg, random_tensors(cfg, seed))
+    reqs = _requests(cfg["vocab"], (330, 37, 150, 2, 90), seed=seed)
+    ref = _reference(folder, reqs)
+    for cut in ("whole", "mixed"):
+        trace = CUTS[cut](reqs)
+        out = str(tmp_path / cut)
+        traces.run_in_process(trace, folder, "float32", out, 16)
+        bad, worst = traces.first_mismatch(traces.collect(trace, out, cfg["vocab"]), ref, 3e-4)
+        assert bad is None, f"{cut}: first wrong logits at (request, position, relative error) {bad}"
 
 
 def test_the_command_line_with_random_weights(tmp_path, capsys):
